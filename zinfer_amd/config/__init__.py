@@ -5,8 +5,11 @@ from .specs import (GatedExpertSpec, LayerNormSpec, MoeSpec, SandwichNormBlockSp
                     TiedKeyValueAttentionSpec)
 from .specs import (DenseMlpSpec, LatentAttentionSpec, LeadingRotarySpec, MaskedGqaAttentionSpec,
                     PostNormBlockSpec)
+from .specs import (GatedLinearAttentionSpec, ParallelBlockSpec, PlainExpertSpec,
+                    SinusoidalPositionSpec, TokenShiftRecurrenceSpec)
 from .specs import (GqaAttentionSpec, ModelSpec, NoPositionSpec, PreNormBlockSpec, RmsNormSpec,
                     RotaryHalfSplitSpec, ScheduleEntry, SwiGluSpec)
 from .qwen3 import Qwen3Config
 from .fezupel import FezupelConfig
 from .lodenex import LodenexConfig
+from .nupovik import NupovikConfig

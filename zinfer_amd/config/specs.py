@@ -135,13 +135,16 @@ class LatentAttentionSpec:
     plain key is W_uk latent and the value W_uv latent; the score is scale * (q_plain . k_plain
     + q_rot . k_rot).  The cache holds the latent and the rotated part only.  ``window`` /
     ``chunk`` as in ``MaskedGqaAttentionSpec``; ``element_gate``: the concatenated heads are
-    multiplied by sigmoid(W_g h) before the output projection."""
+    multiplied by sigmoid(W_g h) before the output projection; ``head_gate``: head h's output
+    is multiplied by sigmoid(W_g h)_h, one number a head (W_g is then [heads, hidden]).
+    ``q_rank`` None: no query latent, q = W_q h with the matrix ``uq_name`` [heads * (head_dim +
+    rot_dim), hidden].  ``rot_dim`` 0: no rotated part, the key is the latent alone."""
     hidden_size: int
     n_heads: int
     head_dim: int
     rot_dim: int
     value_dim: int
-    q_rank: int
+    q_rank: Optional[int]
     kv_rank: int
     scale: float
     norm_eps: float
@@ -149,6 +152,7 @@ class LatentAttentionSpec:
     window: Optional[int] = None
     chunk: Optional[int] = None
     element_gate: bool = False
+    head_gate: bool = False
     dq_name: str = "q_a_proj.weight"
     dq_norm_name: str = "q_a_layernorm.weight"
     uq_name: str = "q_b_proj.weight"
@@ -163,12 +167,76 @@ class LatentAttentionSpec:
 @dataclass(frozen=True)
 class DenseMlpSpec:
     """down(act(up(x))), no gate: ``activation`` is "gelu" (the exact form with erf),
-    "gelu_tanh" or "silu"."""
+    "gelu_tanh", "silu" or "relu2" (the square of max(x, 0))."""
     hidden_size: int
     intermediate_size: int
     activation: str = "gelu"
     up_name: str = "up_proj.weight"
     down_name: str = "down_proj.weight"
+
+
+@dataclass(frozen=True)
+class GatedLinearAttentionSpec:
+    """A mixer whose memory is one matrix a head, S [head_dim, value_dim], carried from token to
+    token in 32-bit: S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with
+    q = W_q h * ``q_scale`` (None: head_dim^(-1/2)), k = W_k h, v = W_v h and a decay a key
+    channel a_t = sigmoid(W_a2 (W_a1 h) + b)^(1 / tau) through a narrow middle of ``decay_rank``.
+    Each head's o goes through an RMS norm over value_dim with one gain for all heads, the heads
+    side by side are multiplied by silu(W_g h), then W_o.  The ``*_name`` fields are the tensor
+    names below the mixer's prefix."""
+    hidden_size: int
+    n_heads: int
+    head_dim: int
+    value_dim: int
+    decay_rank: Optional[int]          # None: whatever the tensors hold
+    tau: float
+    norm_eps: float
+    q_scale: Optional[float] = None
+    q_name: str = "q"
+    k_name: str = "k"
+    v_name: str = "v"
+    gate_name: str = "g"
+    o_name: str = "o"
+    norm_name: str = "norm"
+    decay_down_name: str = "a1"
+    decay_up_name: str = "a2"
+    decay_bias_name: str = "a2.b"
+
+
+@dataclass(frozen=True)
+class TokenShiftRecurrenceSpec:
+    """A mixer of the same kind whose inputs are blends of a token's row with the row before it:
+    m_s = h + (h_prev - h) * mu_s for s in r, k, v, g, w (h_prev zero for a sequence's first
+    token; the last row is part of the state).  r, k, v = W_s m_s (heads of ``head_dim``),
+    gate = silu(W_g m_g), decay w = exp(-exp(W_w2 tanh(W_w1 m_w) + w0)) a head and key channel.
+    o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t with a learned u [heads, head_dim] for the token's
+    own outer product; then S_t = diag(w_t) S_(t-1) + k_t v_t^T.  Each head's o is divided by its
+    root mean square; the heads side by side are multiplied by a gain [heads * head_dim] and the
+    gate, then W_o.  The ``*_name`` fields are the tensor names below the mixer's prefix
+    (``mix_name.format(s)`` for the blends' coefficients)."""
+    hidden_size: int
+    n_heads: int
+    head_dim: int
+    decay_rank: Optional[int]          # None: whatever the tensors hold
+    norm_eps: float
+    r_name: str = "r"
+    k_name: str = "k"
+    v_name: str = "v"
+    gate_name: str = "g"
+    o_name: str = "o"
+    norm_name: str = "norm"
+    bonus_name: str = "u"
+    decay_down_name: str = "w1"
+    decay_up_name: str = "w2"
+    decay_bias_name: str = "w0"
+    mix_name: str = "mu.{}"
+
+
+@dataclass(frozen=True)
+class PlainExpertSpec:
+    """down(act(up(x))), no gate and no bias; ``activation`` as in ``DenseMlpSpec``."""
+    intermediate_size: int
+    activation: str = "relu2"
 
 
 @dataclass(frozen=True)
@@ -185,15 +253,24 @@ class GatedExpertSpec:
 class MoeSpec:
     """Of ``n_experts`` experts every token uses the ``top_k`` whose router logits
     z = W_r x (+ b_r) are largest, weighted by the soft-max over those logits alone; an
-    optional ``shared`` expert runs for every token with weight 1.  Tensor names below the
-    part's prefix: the router's matrix and bias, ``expert_prefix.format(e)`` and
-    ``shared_prefix`` followed by the three matrices' names."""
+    optional ``shared`` expert runs for every token with weight 1.  ``scoring`` "sigmoid"
+    instead: the scores are s = sigmoid(z), the choice goes by s plus a learned correction
+    [n_experts] (``correction_name``; None: none) that does not enter the weights, and the
+    weights are the chosen experts' s over their sum (+ 1e-20); with ``groups`` = (count, keep)
+    the experts form ``count`` equal groups of neighbours, a group is marked by the sum of its
+    two largest choice scores, and only experts of the ``keep`` best groups can be chosen.
+    ``expert`` is a ``GatedExpertSpec`` or a ``PlainExpertSpec`` (no gate matrix).  Tensor names
+    below the part's prefix: the router's matrix and bias, ``expert_prefix.format(e)`` and
+    ``shared_prefix`` followed by the matrices' names."""
     hidden_size: int
     n_experts: int
     top_k: int
-    expert: GatedExpertSpec
+    expert: object
     shared: Optional[GatedExpertSpec] = None
     router_bias: bool = False
+    scoring: str = "softmax"
+    correction_name: Optional[str] = None
+    groups: Optional[Tuple[int, int]] = None
     router_name: str = "gate.weight"
     router_bias_name: str = "gate.bias"
     expert_prefix: str = "experts.{}."
@@ -259,12 +336,37 @@ class PostNormBlockSpec:
 
 
 @dataclass(frozen=True)
+class ParallelBlockSpec:
+    """x += mixer(norm1(x)) + ff(norm2(x)): both sublayers read the same x, each through a norm
+    of its own.  ``feed_forward`` None: the layer is its mixer alone (and declares no
+    ``ff_norm``)."""
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_norm: object
+    ff_norm: Optional[object] = None
+    mixer_prefix: str = "self_attn."
+    ff_prefix: str = "mlp."
+    mixer_norm_prefix: str = "input_layernorm."
+    ff_norm_prefix: str = "post_attention_layernorm."
+
+
+@dataclass(frozen=True)
+class SinusoidalPositionSpec:
+    """A position vector added to the embedding row, formed from the position where it is used:
+    entry 2i is sin(p * f_i), entry 2i + 1 cos(p * f_i), f_i = base^(-2i / width)."""
+    base: float = 10000.0
+
+
+@dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer.  ``layer`` indexes ``ModelSpec.layers`` (a layer may be named
     twice); ``cache_of`` None gives this run a cache of its own, an integer makes it read
-    the cache that the run at that earlier schedule position writes."""
+    the cache that the run at that earlier schedule position writes.  ``reentry``: before this
+    run the stream is replaced by W [x ; x0], x0 being the stream as the embedding left it and W
+    the model's ``reentry_name`` tensor [hidden, 2 hidden] (a pass over looped layers begins)."""
     layer: int
     cache_of: Optional[int] = None
+    reentry: bool = False
 
 
 @dataclass(frozen=True)
@@ -290,3 +392,7 @@ class ModelSpec:
     # a learned position table [max_positions, hidden]: its row at a token's position is added
     # to the embedding row (not scaled); None: positions enter through the mixers only
     position_table_name: Optional[str] = None
+    # a position vector computed from the position and added to the embedding row
+    sinusoidal_positions: Optional[SinusoidalPositionSpec] = None
+    # the matrix [hidden, 2 hidden] of the schedule entries that say ``reentry``
+    reentry_name: Optional[str] = None

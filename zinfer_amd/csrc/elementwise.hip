@@ -29,6 +29,62 @@ extern "C" int zf_embed(const void* table, int table_dtype, const int* ids, floa
   ZF_CHECK_LAUNCH();
 }
 
+// ---------------------------------------------------------------- embedding plus a computed position vector
+// x[t, 2i] = E[id[t], 2i] + sin(p f_i), x[t, 2i + 1] = E[id[t], 2i + 1] + cos(p f_i) with
+// p = positions[t] and the angle p * f_i formed in 32-bit; freq [ceil(H / 2)] float32
+template <typename TW>
+__global__ void embed_sinusoid_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
+                                      const int* __restrict__ positions,
+                                      const float* __restrict__ freq, float* __restrict__ out,
+                                      int H, float scale) {
+  const int t = blockIdx.x;
+  const TW* row = table + (size_t)ids[t] * H;
+  float* o = out + (size_t)t * H;
+  const float p = (float)positions[t];
+  for (int i = threadIdx.x; i < (H + 1) / 2; i += blockDim.x) {
+    float sn, cs;
+    sincosf(p * freq[i], &sn, &cs);
+    o[2 * i] = load_as_float<TW>(row + 2 * i) * scale + sn;
+    if (2 * i + 1 < H) o[2 * i + 1] = load_as_float<TW>(row + 2 * i + 1) * scale + cs;
+  }
+}
+
+extern "C" int zf_embed_sinusoid(const void* table, int table_dtype, const int* ids,
+                                 const int* positions, const float* freq, float* out, int T,
+                                 int H, float scale, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (table_dtype == ZF_F32)
+    hipLaunchKernelGGL(embed_sinusoid_kernel<float>, dim3(T), dim3(256), 0, stream,
+                       (const float*)table, ids, positions, freq, out, H, scale);
+  else
+    hipLaunchKernelGGL(embed_sinusoid_kernel<bf16_t>, dim3(T), dim3(256), 0, stream,
+                       (const bf16_t*)table, ids, positions, freq, out, H, scale);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- two streams side by side
+// out[t, :] = [a[t, :] | b[t, :]] in out's type: what a product over both streams reads
+template <typename TO>
+__global__ void concat_rows_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                   TO* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < 2 * H; i += blockDim.x)
+    store_from_float<TO>(out + (size_t)t * 2 * H + i,
+                         i < H ? a[(size_t)t * H + i] : b[(size_t)t * H + i - H]);
+}
+
+extern "C" int zf_concat_rows(const float* a, const float* b, void* out, int out_dtype, int T,
+                              int H, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (out_dtype == ZF_F32)
+    hipLaunchKernelGGL(concat_rows_kernel<float>, dim3(T), dim3(256), 0, stream, a, b,
+                       (float*)out, H);
+  else
+    hipLaunchKernelGGL(concat_rows_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, a, b,
+                       (bf16_t*)out, H);
+  ZF_CHECK_LAUNCH();
+}
+
 // ---------------------------------------------------------------- logits after the head
 // x = x * scale, then, with cap > 0, x = cap * tanh(x / cap): what an architecture may ask for
 // between the head's product and the sampler
@@ -499,15 +555,9 @@ extern "C" int zf_swiglu(const void* gu, void* out, int dtype, int T, int I,
 
 // ---------------------------------------------------------------- an activation alone, in place or not
 // kind 0: gelu(z) = z/2 (1 + erf(z / sqrt 2));  kind 1: its tanh form
-// z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));  kind 2: silu(z) = z / (1 + exp(-z)).
+// z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));  kind 2: silu(z) = z / (1 + exp(-z));
+// kind 3: max(z, 0)^2;  kind 4: tanh(z).
 // 32-bit arithmetic on values of either storage type.
-__device__ __forceinline__ float activation_value(float z, int kind) {
-  if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
-  if (kind == 1)
-    return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
-  return z / (1.0f + expf(-z));
-}
-
 template <typename T>
 __global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n,
                                   int kind) {
@@ -519,7 +569,7 @@ __global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, 
 extern "C" int zf_activation(const void* x, void* out, int dtype, long long n, int kind,
                              hipStream_t stream) {
   if (n <= 0) return 0;
-  if (kind < 0 || kind > 2) return -2;
+  if (kind < 0 || kind > 4) return -2;
   const unsigned blocks = (unsigned)((n + 255) / 256);
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(activation_kernel<float>, dim3(blocks), dim3(256), 0, stream,

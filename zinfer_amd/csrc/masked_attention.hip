@@ -993,11 +993,14 @@ __global__ __launch_bounds__(ZF_WAVE) void masked_attention_merge_kernel(
                      ws_o, ws_ml, a)
 
 // the shapes that are built: values of their own as wide as the keys; and the keys' leading
-// columns as values (a latent and a rotated part behind it)
+// columns as values (a latent and a rotated part behind it, or the latent alone)
 #define MW_SHAPES(DEC)                                                                           \
   if (!tied && KD == 64 && VD == 64) MW_LAUNCH(64, 64, false, DEC);                              \
   else if (!tied && KD == 96 && VD == 96) MW_LAUNCH(96, 96, false, DEC);                         \
   else if (!tied && KD == 128 && VD == 128) MW_LAUNCH(128, 128, false, DEC);                     \
+  else if (tied && KD == 64 && VD == 64) MW_LAUNCH(64, 64, true, DEC);                           \
+  else if (tied && KD == 96 && VD == 96) MW_LAUNCH(96, 96, true, DEC);                           \
+  else if (tied && KD == 128 && VD == 128) MW_LAUNCH(128, 128, true, DEC);                       \
   else if (tied && KD == 96 && VD == 64) MW_LAUNCH(96, 64, true, DEC);                           \
   else if (tied && KD == 160 && VD == 128) MW_LAUNCH(160, 128, true, DEC);                       \
   else if (tied && KD == 192 && VD == 128) MW_LAUNCH(192, 128, true, DEC);                       \

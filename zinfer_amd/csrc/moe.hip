@@ -1,10 +1,14 @@
 // A feed-forward layer made of many small experts, of which every token uses a few.
 //
 //   router:  z = R h + r            32-bit; the `top` largest z are chosen (the lower index
-//            wins a tie), and their weights are the soft-max over the chosen z alone
+//            wins a tie), and their weights are the soft-max over the chosen z alone;
+//            or (scoring 1) s = sigmoid(z), the choice goes by s + correction among the experts
+//            of the best groups (a group of neighbours is marked by its two largest choice
+//            scores added), and the weights are the chosen s over their sum (+ 1e-20)
 //   expert:  g = min(Wg h, limit), u = clamp(Wu h, -limit, limit)      (limit <= 0: no clamp)
 //            y = g * sigmoid(alpha * g) * (u + shift)
 //            out = Wd y
+//            or, without a gate: y = act(Wu h) with one of the plain activations
 //   layer:   out[t] = sum over the chosen experts of weight * expert(h[t])
 //
 // Expert matrices are stacked: gate_up [E, 2 * ff, W] (an expert's gate rows, then its up
@@ -48,9 +52,11 @@ template <> struct Vec4<bf16_t> {
 template <typename T>
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ router, const float* __restrict__ bias,
-    int* __restrict__ ids, float* __restrict__ weights, int n_tokens, int W, int E, int top) {
+    int* __restrict__ ids, float* __restrict__ weights, int n_tokens, int W, int E, int top,
+    int scoring, const float* __restrict__ correction, int n_groups, int keep_groups) {
   __shared__ float zs[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS], shares[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
   __shared__ int chosens[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
+  __shared__ unsigned char kepts[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
   const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
   const int t0 = blockIdx.x * MOE_ROUTE_TOKENS;
   const T* rows[MOE_ROUTE_TOKENS];
@@ -96,6 +102,85 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
   float* z = zs[wave];
   float* share = shares[wave];
   int* chosen = chosens[wave];
+  if (scoring == 1) {
+    // scores s = sigmoid(z) (kept in `share`), choice scores s + correction (in `z`)
+    for (int e = lane; e < E; e += ZF_WAVE) {
+      const float sc = 1.0f / (1.0f + expf(-z[e]));
+      share[e] = sc;
+      z[e] = sc + (correction != nullptr ? correction[e] : 0.f);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    if (n_groups > 0 && keep_groups < n_groups) {
+      // a group's mark: its two largest choice scores added (its one score, if it has one)
+      float* mark = (float*)chosen;
+      unsigned char* kept = kepts[wave];
+      const int size = E / n_groups;
+      for (int g = lane; g < n_groups; g += ZF_WAVE) {
+        float a = -INFINITY, b = -INFINITY;
+        for (int e = g * size; e < (g + 1) * size; ++e) {
+          const float v = z[e];
+          if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+        }
+        mark[g] = size > 1 ? a + b : a;
+        kept[g] = 0;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_wave_barrier();
+      for (int k = 0; k < keep_groups; ++k) {
+        float best = -INFINITY;
+        int arg = 0x7fffffff;
+        for (int g = lane; g < n_groups; g += ZF_WAVE) {
+          const float v = mark[g];
+          if (!kept[g] && (v > best || arg == 0x7fffffff)) { best = v; arg = g; }
+        }
+#pragma unroll
+        for (int off = ZF_WAVE / 2; off > 0; off >>= 1) {
+          const float ob = __shfl_xor(best, off, ZF_WAVE);
+          const int oa = __shfl_xor(arg, off, ZF_WAVE);
+          if (oa != 0x7fffffff && (arg == 0x7fffffff || ob > best || (ob == best && oa < arg))) {
+            best = ob; arg = oa;
+          }
+        }
+        if (lane == 0 && arg != 0x7fffffff) kept[arg] = 1;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+      }
+      // outside the kept groups nothing can be chosen
+      for (int e = lane; e < E; e += ZF_WAVE)
+        if (!kept[e / size]) z[e] = -INFINITY;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_wave_barrier();
+    }
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+      float best = -INFINITY;
+      int arg = 0x7fffffff;
+      for (int e = lane; e < E; e += ZF_WAVE) {
+        const float v = z[e];
+        if (v > best) { best = v; arg = e; }
+      }
+#pragma unroll
+      for (int off = ZF_WAVE / 2; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, ZF_WAVE);
+        const int oa = __shfl_xor(arg, off, ZF_WAVE);
+        if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
+      }
+      if (arg == 0x7fffffff) arg = 0;
+      sum += share[arg];
+      if (lane == 0) {
+        chosen[k] = arg;
+        z[arg] = -INFINITY;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_wave_barrier();
+    }
+    for (int k = lane; k < top; k += ZF_WAVE) {
+      ids[(size_t)t * top + k] = chosen[k];
+      weights[(size_t)t * top + k] = share[chosen[k]] / (sum + 1e-20f);
+    }
+    return;
+  }
   // `top` rounds of: the largest remaining logit, the lowest index among equals
   float first = 0.f, sum = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -131,16 +216,23 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
 
 extern "C" int zf_moe_route(const void* h, int dtype, const float* router, const float* bias,
                             int* ids, float* weights, int T, int W, int E, int top,
+                            int scoring, const float* correction, int n_groups, int keep_groups,
                             hipStream_t stream) {
   if (T <= 0) return 0;
-  if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E) return -2;
+  if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E || scoring < 0 || scoring > 1 ||
+      n_groups < 0 || (n_groups > 0 && (E % n_groups != 0 || keep_groups < 1 ||
+                                        keep_groups > n_groups ||
+                                        top > keep_groups * (E / n_groups))))
+    return -2;
   const dim3 grid((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS), block(MOE_ROUTE_WAVES * ZF_WAVE);
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, 0, stream, (const float*)h, router,
-                       bias, ids, weights, T, W, E, top);
+                       bias, ids, weights, T, W, E, top, scoring, correction, n_groups,
+                       keep_groups);
   else
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, router,
-                       bias, ids, weights, T, W, E, top);
+                       bias, ids, weights, T, W, E, top, scoring, correction, n_groups,
+                       keep_groups);
   ZF_CHECK_LAUNCH();
 }
 
@@ -206,10 +298,12 @@ __device__ __forceinline__ float row_dot(const T* __restrict__ w, const T* __res
 #define MOE_WAVES 4
 #define MOE_GU_PER_WAVE 4      // outputs of y a wave computes, one after the other
 
-template <typename T>
+// GATED: gate_up [E, 2 ff, W] and the gated activation; else `gate_up` holds the up rows alone,
+// [E, ff, W], and y = activation_value(up, act) (`act` by the numbers of zf_common.h).
+template <typename T, bool GATED>
 __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_gate_up_kernel(
     const T* __restrict__ h, const T* __restrict__ gate_up, const int* __restrict__ ids,
-    T* __restrict__ y, int W, int ff, int slots, float limit, float alpha, float shift) {
+    T* __restrict__ y, int W, int ff, int slots, float limit, float alpha, float shift, int act) {
   extern __shared__ float xs[];                    // the token's row, [W]
   const int ts = blockIdx.x, t = ts / slots;
   const int e = ids != nullptr ? ids[ts] : 0;
@@ -217,7 +311,7 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_gate_up_kernel(
   const T* row = h + (size_t)t * W;
   for (int i = threadIdx.x; i < W; i += blockDim.x) xs[i] = load_as_float<T>(row + i);
   __syncthreads();
-  const T* we = gate_up + (size_t)e * 2 * ff * W;
+  const T* we = gate_up + (size_t)e * (GATED ? 2 : 1) * ff * W;
   const int j0 = (blockIdx.y * MOE_WAVES + wave) * MOE_GU_PER_WAVE;
   if (j0 >= ff) return;
   if constexpr (sizeof(T) == 2) {
@@ -237,56 +331,72 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_gate_up_kernel(
 #pragma unroll
         for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
           a[o] = *(const uint4*)(gr[o] + i);
-          b[o] = *(const uint4*)(gr[o] + (size_t)ff * W + i);
+          if constexpr (GATED) b[o] = *(const uint4*)(gr[o] + (size_t)ff * W + i);
         }
         const float4 x0 = *(const float4*)(xs + i), x1 = *(const float4*)(xs + i + 4);
         const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
 #pragma unroll
         for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
           const uint32_t p[4] = {a[o].x, a[o].y, a[o].z, a[o].w};
-          const uint32_t q[4] = {b[o].x, b[o].y, b[o].z, b[o].w};
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
             dg[o] = fmaf(__uint_as_float(p[c] << 16), x[2 * c], dg[o]);
             dg[o] = fmaf(__uint_as_float(p[c] & 0xffff0000u), x[2 * c + 1], dg[o]);
-            du[o] = fmaf(__uint_as_float(q[c] << 16), x[2 * c], du[o]);
-            du[o] = fmaf(__uint_as_float(q[c] & 0xffff0000u), x[2 * c + 1], du[o]);
+          }
+          if constexpr (GATED) {
+            const uint32_t q[4] = {b[o].x, b[o].y, b[o].z, b[o].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              du[o] = fmaf(__uint_as_float(q[c] << 16), x[2 * c], du[o]);
+              du[o] = fmaf(__uint_as_float(q[c] & 0xffff0000u), x[2 * c + 1], du[o]);
+            }
           }
         }
       }
 #pragma unroll
       for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
-        const float g = wave_sum(dg[o]), u = wave_sum(du[o]);
-        if (lane == 0 && j0 + o < ff)
-          store_from_float<T>(y + (size_t)ts * ff + j0 + o, gated_unit(g, u, limit, alpha, shift));
+        const float g = wave_sum(dg[o]);
+        float r;
+        if constexpr (GATED) r = gated_unit(g, wave_sum(du[o]), limit, alpha, shift);
+        else r = activation_value(g, act);
+        if (lane == 0 && j0 + o < ff) store_from_float<T>(y + (size_t)ts * ff + j0 + o, r);
       }
       return;
     }
   }
   for (int j = j0; j < j0 + MOE_GU_PER_WAVE && j < ff; ++j) {
     const float g = wave_sum(row_dot_lds<T>(we + (size_t)j * W, xs, W, lane));
-    const float u = wave_sum(row_dot_lds<T>(we + (size_t)(ff + j) * W, xs, W, lane));
-    if (lane == 0)
-      store_from_float<T>(y + (size_t)ts * ff + j, gated_unit(g, u, limit, alpha, shift));
+    float r;
+    if constexpr (GATED) {
+      const float u = wave_sum(row_dot_lds<T>(we + (size_t)(ff + j) * W, xs, W, lane));
+      r = gated_unit(g, u, limit, alpha, shift);
+    } else {
+      r = activation_value(g, act);
+    }
+    if (lane == 0) store_from_float<T>(y + (size_t)ts * ff + j, r);
   }
 }
 
+// gated != 0: gate_up [E, 2 ff, W]; else [E, ff, W] and the plain activation `act`
 extern "C" int zf_moe_gate_up(const void* h, const void* gate_up, int dtype, const int* ids,
                               void* y, int T, int W, int ff, int slots, float limit, float alpha,
-                              float shift, hipStream_t stream) {
+                              float shift, int gated, int act, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (W <= 0 || ff <= 0 || slots <= 0 || (size_t)W * sizeof(float) > 64 * 1024) return -2;
+  if (W <= 0 || ff <= 0 || slots <= 0 || (size_t)W * sizeof(float) > 64 * 1024 || act < 0 ||
+      act > 4)
+    return -2;
   const int per_wg = MOE_WAVES * MOE_GU_PER_WAVE;
   dim3 grid(T * slots, (ff + per_wg - 1) / per_wg);
   const size_t smem = (size_t)W * sizeof(float);
-  if (dtype == ZF_F32)
-    hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, dim3(MOE_WAVES * ZF_WAVE), smem, stream,
-                       (const float*)h, (const float*)gate_up, ids, (float*)y, W, ff, slots,
-                       limit, alpha, shift);
-  else
-    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, dim3(MOE_WAVES * ZF_WAVE), smem, stream,
-                       (const bf16_t*)h, (const bf16_t*)gate_up, ids, (bf16_t*)y, W, ff, slots,
-                       limit, alpha, shift);
+#define MOE_GU_LAUNCH(TT, G)                                                                      \
+  hipLaunchKernelGGL((moe_gate_up_kernel<TT, G>), grid, dim3(MOE_WAVES * ZF_WAVE), smem, stream, \
+                     (const TT*)h, (const TT*)gate_up, ids, (TT*)y, W, ff, slots, limit, alpha,  \
+                     shift, act)
+  if (dtype == ZF_F32) {
+    if (gated) MOE_GU_LAUNCH(float, true); else MOE_GU_LAUNCH(float, false);
+  } else {
+    if (gated) MOE_GU_LAUNCH(bf16_t, true); else MOE_GU_LAUNCH(bf16_t, false);
+  }
   ZF_CHECK_LAUNCH();
 }
 
@@ -487,13 +597,17 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t moe_u32x
 // of an operand, and of the result column lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4.
 #define MOE_NB 2                 // weight tiles of 64 rows a workgroup holds
 #define MOE_HALF (MOE_NB / 2)
-template <bool GATED>
+// MODE 0: the down pass; 1: gate and up with the gated activation; 2: up alone, w [E, N, K], with
+// the plain activation `act`.
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ a, long long lda, const int* __restrict__ sorted, int top,
     const bf16_t* __restrict__ w, const int* __restrict__ tile_expert,
     const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
     const int* __restrict__ n_tiles, void* __restrict__ out, int N, int K, float limit,
-    float alpha, float shift) {
+    float alpha, float shift, int act) {
+  constexpr bool GATED = MODE == 1;
+  constexpr bool GATHER = MODE != 0;            // rows of h found through the sort
   __shared__ __attribute__((aligned(16))) bf16_t as[MOE_TILE_ROWS * MOE_LD];
   __shared__ __attribute__((aligned(16))) bf16_t bs[MOE_NB * 64 * MOE_LD];
   // gridDim.x is a multiple of 8: workgroup x takes tile (x % 8) * (gridDim.x / 8) + x / 8, so
@@ -515,7 +629,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const int r = sr + 32 * i;
     ap[i] = nullptr;
     if (r < nrows) {
-      const int src = GATED ? sorted[row0 + r] / top : row0 + r;
+      const int src = GATHER ? sorted[row0 + r] / top : row0 + r;
       ap[i] = a + (size_t)src * lda;
     }
   }
@@ -593,6 +707,12 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
           if (c0 + j * 64 + col < N)
             ((bf16_t*)out)[(size_t)(row0 + row) * N + c0 + j * 64 + col] =
                 float_to_bf16(gated_unit(acc[i][j][r], acc[i][MOE_HALF + j][r], limit, alpha, shift));
+      } else if (MODE == 2) {
+#pragma unroll
+        for (int j = 0; j < MOE_NB; ++j)
+          if (c0 + j * 64 + col < N)
+            ((bf16_t*)out)[(size_t)(row0 + row) * N + c0 + j * 64 + col] =
+                float_to_bf16(activation_value(acc[i][j][r], act));
       } else {
 #pragma unroll
         for (int j = 0; j < MOE_NB; ++j)
@@ -602,24 +722,26 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     }
 }
 
-// GATED: a = h [T, K] (rows gathered), w = gate_up [E, 2 N, K], out = y bfloat16 [P, N];
-// else a = y [P, K], w = down [E, N, K], out = o float32 [P, N].  K a multiple of 8.
+// mode 1: a = h [T, K] (rows gathered), w = gate_up [E, 2 N, K], out = y bfloat16 [P, N];
+// mode 2: the same with w = up [E, N, K] and the plain activation `act`;
+// mode 0: a = y [P, K], w = down [E, N, K], out = o float32 [P, N].  K a multiple of 8.
 extern "C" int zf_moe_grouped(const void* a, long long lda, const int* sorted, int top,
                               const void* w, const int* tile_expert, const int* tile_row0,
                               const int* tile_rows, const int* n_tiles, void* out, int max_tiles,
-                              int N, int K, int gated, float limit, float alpha, float shift,
-                              hipStream_t stream) {
+                              int N, int K, int mode, float limit, float alpha, float shift,
+                              int act, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
-  if (N <= 0 || K <= 0 || K % 8 != 0 || top <= 0) return -2;
+  if (N <= 0 || K <= 0 || K % 8 != 0 || top <= 0 || mode < 0 || mode > 2 || act < 0 || act > 4)
+    return -2;
   max_tiles = (max_tiles + 7) / 8 * 8;
-  if (gated)
-    hipLaunchKernelGGL(moe_grouped_kernel<true>, dim3(max_tiles, (N + 64 * MOE_HALF - 1) / (64 * MOE_HALF)), dim3(256), 0,
-                       stream, (const bf16_t*)a, lda, sorted, top, (const bf16_t*)w, tile_expert,
-                       tile_row0, tile_rows, n_tiles, out, N, K, limit, alpha, shift);
-  else
-    hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(max_tiles, (N + 64 * MOE_NB - 1) / (64 * MOE_NB)), dim3(256), 0,
-                       stream, (const bf16_t*)a, lda, sorted, top, (const bf16_t*)w, tile_expert,
-                       tile_row0, tile_rows, n_tiles, out, N, K, limit, alpha, shift);
+#define MOE_GROUPED_LAUNCH(MODE, COLS)                                                           \
+  hipLaunchKernelGGL(moe_grouped_kernel<MODE>, dim3(max_tiles, (N + (COLS) - 1) / (COLS)),       \
+                     dim3(256), 0, stream, (const bf16_t*)a, lda, sorted, top, (const bf16_t*)w, \
+                     tile_expert, tile_row0, tile_rows, n_tiles, out, N, K, limit, alpha, shift, \
+                     act)
+  if (mode == 1) MOE_GROUPED_LAUNCH(1, 64 * MOE_HALF);
+  else if (mode == 2) MOE_GROUPED_LAUNCH(2, 64 * MOE_NB);
+  else MOE_GROUPED_LAUNCH(0, 64 * MOE_NB);
   ZF_CHECK_LAUNCH();
 }
 

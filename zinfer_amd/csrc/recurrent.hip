@@ -1,0 +1,264 @@
+// Mixers whose memory of a sequence is a matrix of fixed size a head, carried from token to
+// token in 32-bit, instead of a cache that grows:
+//
+//   S_t = diag(a_t) S_(t-1) + k_t v_t^T          S is [d, dv] a head, a_t in (0, 1) a key channel
+//   after:   o_t = S_t^T q_t                     (the output reads the new state)
+//   before:  o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t      (the old state, and the token's own
+//                                                 outer product weighted by a learned u)
+//
+// The decay a_t comes from 32-bit numbers z_t (a projection's output) by one of two rules:
+//   rule 0:  a = sigmoid(z + b)^(1 / tau) = exp(-softplus(-(z + b)) / tau)
+//   rule 1:  a = exp(-exp(z + b))
+// Everything but the rows q, k, v themselves is 32-bit in both storage types.
+//
+//  * token_shift_mix     m_s[t] = h[t] + (h[t-1] - h[t]) * mu_s for several s at once; the row
+//                        before a portion's first is the request's state (zero at the start),
+//                        which then takes the portion's last row
+//  * decay_recurrence    the recurrence, token by token; a request's state is read at the start
+//                        of its portion and written at its end
+//  * head_norm_gate      out = o / rms_head(o) * gain * silu(g)
+#include "zf_common.h"
+
+// ---------------------------------------------------------------- token shift
+// grid (token), any block: mixes [n_mix][T][W] in the rows' type.  The workgroup of a portion's
+// first token reads the state row and is the one that overwrites it (with the portion's last
+// row), element by element in the thread that read it: no other workgroup touches that row.
+template <typename T>
+__global__ void token_shift_mix_kernel(const T* __restrict__ h, const float* __restrict__ mu,
+                                       float* __restrict__ state, long long slot_stride,
+                                       const int* __restrict__ state_slots,
+                                       const int* __restrict__ seq_index,
+                                       const int* __restrict__ q_start, T* __restrict__ out,
+                                       int n_tokens, int W, int n_mix) {
+  const int t = blockIdx.x;
+  const int s = seq_index[t];
+  const int t0 = q_start[s], t1 = q_start[s + 1];
+  const bool first = t == t0;
+  const T* row = h + (size_t)t * W;
+  const T* before = first ? nullptr : row - W;
+  float* st = state + (size_t)state_slots[s] * slot_stride;
+  const T* last = h + (size_t)(t1 - 1) * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float x = load_as_float<T>(row + i);
+    const float p = first ? st[i] : load_as_float<T>(before + i);
+    const float dx = p - x;
+    for (int m = 0; m < n_mix; ++m)
+      store_from_float<T>(out + ((size_t)m * n_tokens + t) * W + i,
+                          fmaf(dx, mu[(size_t)m * W + i], x));
+    if (first) st[i] = load_as_float<T>(last + i);
+  }
+}
+
+extern "C" int zf_token_shift_mix(const void* h, int dtype, const float* mu, float* state,
+                                  long long slot_stride, const int* state_slots,
+                                  const int* seq_index, const int* q_start, void* out, int T,
+                                  int W, int n_mix, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (W <= 0 || n_mix <= 0) return -2;
+  const int block = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+  if (dtype == ZF_F32)
+    hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(T), dim3(block), 0, stream,
+                       (const float*)h, mu, state, slot_stride, state_slots, seq_index, q_start,
+                       (float*)out, T, W, n_mix);
+  else
+    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, dim3(T), dim3(block), 0, stream,
+                       (const bf16_t*)h, mu, state, slot_stride, state_slots, seq_index, q_start,
+                       (bf16_t*)out, T, W, n_mix);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- the recurrence
+#define REC_R 8            // key channels of a value column a thread keeps in registers
+#define REC_TC 16          // tokens staged at a time (half of that for more than 128 channels)
+#define REC_MAX_THREADS 256
+
+__device__ __forceinline__ float decay_of(float z, int rule, float inv_tau) {
+  if (rule == 0) {
+    // log sigmoid(z) = -softplus(-z)
+    const float x = -z;
+    const float sp = fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
+    return expf(-sp * inv_tau);
+  }
+  return expf(-expf(z));
+}
+
+// grid (sequence, head, block of VB value columns); thread (vl, cg) = (tid / CS, tid % CS)
+// holds S[8 cg .. 8 cg + 8, v0 + vl].  A request's state is laid out [head][dv][CS * 8]: the
+// channels a thread holds lie side by side (channels beyond d are padding that stays zero).
+// A token's partial outputs (one a thread) go to LDS and are added in ascending cg, so the sum
+// over channels has one order whatever VB is and however a prompt is cut.
+template <typename T, bool BEFORE>
+__global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
+    const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride,
+    const T* __restrict__ v, long long v_stride, const float* __restrict__ z,
+    const float* __restrict__ z_bias, const float* __restrict__ bonus,
+    float* __restrict__ state, long long slot_stride, const int* __restrict__ state_slots,
+    const int* __restrict__ q_start, float* __restrict__ out, int H, int d, int dv, int CS,
+    int VB, int TC, int rule, float inv_tau, float q_scale) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int DP = CS * REC_R;
+  float* qs = lds;                        // [TC][DP]
+  float* ks = qs + TC * DP;               // [TC][DP]
+  float* ds = ks + TC * DP;               // [TC][DP]
+  float* us = ds + TC * DP;               // [DP]
+  float* vs = us + DP;                    // [TC][VB]
+  float* po = vs + TC * VB;               // [TC][VB][CS]
+  const int s = blockIdx.x, hd = blockIdx.y, v0 = blockIdx.z * VB;
+  const int t0 = q_start[s], t1 = q_start[s + 1];
+  if (t0 >= t1) return;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int vl = tid / CS, cg = tid % CS;
+  const bool mine = vl < VB && v0 + vl < dv;
+  float* st = state + (size_t)state_slots[s] * slot_stride +
+              ((size_t)hd * dv + v0 + vl) * DP + cg * REC_R;
+  float S[REC_R];
+#pragma unroll
+  for (int j = 0; j < REC_R; ++j) S[j] = 0.f;
+  if (mine) {
+    const float4 a = *(const float4*)st, b = *(const float4*)(st + 4);
+    S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w;
+    S[4] = b.x; S[5] = b.y; S[6] = b.z; S[7] = b.w;
+  }
+  for (int c = tid; c < DP; c += nthreads)
+    us[c] = (BEFORE && c < d) ? bonus[hd * d + c] : 0.f;
+  for (int tc = t0; tc < t1; tc += TC) {
+    const int n = min(TC, t1 - tc);
+    __syncthreads();                      // the chunk before is read and reduced
+    for (int i = tid; i < n * DP; i += nthreads) {
+      const int t = i / DP, c = i % DP;
+      float qv = 0.f, kv = 0.f, dc = 1.f;
+      if (c < d) {
+        const size_t row = (size_t)(tc + t);
+        qv = load_as_float<T>(q + row * q_stride + hd * d + c) * q_scale;
+        kv = load_as_float<T>(k + row * k_stride + hd * d + c);
+        dc = decay_of(z[row * ((size_t)H * d) + hd * d + c] + z_bias[hd * d + c], rule, inv_tau);
+      }
+      qs[i] = qv; ks[i] = kv; ds[i] = dc;
+    }
+    for (int i = tid; i < n * VB; i += nthreads) {
+      const int t = i / VB, x = i % VB;
+      vs[i] = v0 + x < dv ? load_as_float<T>(v + (size_t)(tc + t) * v_stride + hd * dv + v0 + x)
+                          : 0.f;
+    }
+    __syncthreads();
+    if (vl < VB) {
+      for (int t = 0; t < n; ++t) {
+        const float vv = vs[t * VB + vl];
+        const float4* qp = (const float4*)(qs + t * DP + cg * REC_R);
+        const float4* kp = (const float4*)(ks + t * DP + cg * REC_R);
+        const float4* dp = (const float4*)(ds + t * DP + cg * REC_R);
+        const float4 q0 = qp[0], q1 = qp[1], k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
+        const float q8[REC_R] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const float k8[REC_R] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        const float d8[REC_R] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+        float acc = 0.f;
+        if (BEFORE) {
+          const float4* up = (const float4*)(us + cg * REC_R);
+          const float4 u0 = up[0], u1 = up[1];
+          const float u8[REC_R] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+          for (int j = 0; j < REC_R; ++j) {
+            const float kv = k8[j] * vv;
+            acc = fmaf(q8[j], fmaf(u8[j], kv, S[j]), acc);
+            S[j] = fmaf(d8[j], S[j], kv);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < REC_R; ++j) {
+            S[j] = fmaf(d8[j], S[j], k8[j] * vv);
+            acc = fmaf(q8[j], S[j], acc);
+          }
+        }
+        po[(t * VB + vl) * CS + cg] = acc;
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < n * VB; i += nthreads) {
+      const int t = i / VB, x = i % VB;
+      if (v0 + x >= dv) continue;
+      float sum = 0.f;
+      for (int c = 0; c < CS; ++c) sum += po[i * CS + c];
+      out[(size_t)(tc + t) * ((size_t)H * dv) + hd * dv + v0 + x] = sum;
+    }
+  }
+  if (mine) {
+    *(float4*)st = float4{S[0], S[1], S[2], S[3]};
+    *(float4*)(st + 4) = float4{S[4], S[5], S[6], S[7]};
+  }
+}
+
+// q, k [T, >= H d], v [T, >= H dv] with contiguous rows (strides in elements), z [T, H d] and
+// out [T, H dv] float32, dense.  CS = ceil(d / 8) <= 32; VB value columns a workgroup,
+// CS * VB <= 256.
+extern "C" int zf_decay_recurrence(const void* q, long long q_stride, const void* k,
+                                   long long k_stride, const void* v, long long v_stride,
+                                   int dtype, const float* z, const float* z_bias,
+                                   const float* bonus, float* state, long long slot_stride,
+                                   const int* state_slots, const int* q_start, float* out,
+                                   int n_seqs, int H, int d, int dv, int VB, int rule,
+                                   float inv_tau, float q_scale, hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  const int CS = (d + REC_R - 1) / REC_R;
+  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 || CS * VB > REC_MAX_THREADS ||
+      rule < 0 || rule > 1 || slot_stride < (long long)H * dv * CS * REC_R)
+    return -2;
+  const int DP = CS * REC_R;
+  const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
+  const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + DP + (size_t)TC * VB +
+                                       (size_t)TC * VB * CS);
+  const int threads = (CS * VB + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
+  const dim3 grid(n_seqs, H, (dv + VB - 1) / VB), block(threads);
+#define REC_LAUNCH(TT, BEF)                                                                      \
+  hipLaunchKernelGGL((decay_recurrence_kernel<TT, BEF>), grid, block, smem, stream,              \
+                     (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z,  \
+                     z_bias, bonus, state, slot_stride, state_slots, q_start, out, H, d, dv, CS, \
+                     VB, TC, rule, inv_tau, q_scale)
+  if (dtype == ZF_F32) {
+    if (bonus != nullptr) REC_LAUNCH(float, true); else REC_LAUNCH(float, false);
+  } else {
+    if (bonus != nullptr) REC_LAUNCH(bf16_t, true); else REC_LAUNCH(bf16_t, false);
+  }
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- norm a head, gain, gate
+// a wave a (token, head): out[t, h, :] = o / sqrt(mean(o^2) + eps) * gain * silu(g[t, h, :]);
+// gain [dv] (one for all heads) or [H dv].  o float32, g and out in the rows' type.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(
+    const float* __restrict__ o, const float* __restrict__ gain, int gain_per_head,
+    const T* __restrict__ g, long long g_stride, T* __restrict__ out, int n_rows, int H, int dv,
+    float eps) {
+  const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
+  const int r = blockIdx.x * (blockDim.x / ZF_WAVE) + wave;       // (token, head)
+  if (r >= n_rows) return;
+  const int t = r / H, hd = r % H;
+  const float* row = o + (size_t)r * dv;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += ZF_WAVE) ss = fmaf(row[i], row[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+  const T* gr = g + (size_t)t * g_stride + hd * dv;
+  const float* gn = gain + (gain_per_head ? hd * dv : 0);
+  for (int i = lane; i < dv; i += ZF_WAVE) {
+    const float gv = load_as_float<T>(gr + i);
+    const float silu = gv / (1.0f + expf(-gv));
+    store_from_float<T>(out + (size_t)r * dv + i, row[i] * inv * gn[i] * silu);
+  }
+}
+
+extern "C" int zf_head_norm_gate(const float* o, const float* gain, int gain_per_head,
+                                 const void* g, long long g_stride, void* out, int dtype, int T,
+                                 int H, int dv, float eps, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || dv <= 0) return -2;
+  const int rows = T * H;
+  const dim3 grid((rows + 3) / 4), block(4 * ZF_WAVE);
+  if (dtype == ZF_F32)
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, o, gain,
+                       gain_per_head, (const float*)g, g_stride, (float*)out, rows, H, dv, eps);
+  else
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, o, gain,
+                       gain_per_head, (const bf16_t*)g, g_stride, (bf16_t*)out, rows, H, dv, eps);
+  ZF_CHECK_LAUNCH();
+}

@@ -144,6 +144,17 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return total;
 }
 
+// An activation alone, by number (32-bit arithmetic): 0 gelu(z) = z/2 (1 + erf(z / sqrt 2)),
+// 1 its tanh form, 2 silu(z) = z / (1 + exp(-z)), 3 max(z, 0)^2, 4 tanh(z).
+__device__ __forceinline__ float activation_value(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
+  if (kind == 1)
+    return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+  if (kind == 3) { const float r = fmaxf(z, 0.f); return r * r; }
+  if (kind == 4) return tanhf(z);
+  return z / (1.0f + expf(-z));
+}
+
 // dtype codes shared with the Python side
 #define ZF_F32 0
 #define ZF_BF16 1

@@ -374,8 +374,10 @@ class Engine:
             raise CacheFull("CacheFull: the step needs more pages or request slots than are free")
         added = self._reserve(wanted_len)
         out: Dict[str, float] = {}
+        saved = []
         try:
             ctx = self._build_context(entries, bucket_pages=True)
+            saved = self._save_states(ctx.slots)
             self.model.forward(ctx, self.views)           # settles every work buffer's size
             stream = torch.cuda.current_stream(self.device)
             for cls in ops.KERNEL_CLASSES + ("step",):
@@ -402,8 +404,21 @@ class Engine:
                 out[cls] = before.elapsed_time(after) * 1e-3 / repeats
                 del graph
         finally:
+            self._restore_states(None, saved)
             self._roll_back(wanted_len, added)
         return out
+
+    def _save_states(self, slots):
+        """Copies of the state rows of ``slots`` in every state pool (none: an empty list)."""
+        pools = self.cache.state_pools
+        if not pools:
+            return []
+        index = torch.tensor(list(slots), dtype=torch.long, device=self.device)
+        return [(pool, index, pool.index_select(0, index)) for pool in pools.values()]
+
+    def _restore_states(self, slots, saved) -> None:
+        for pool, index, rows in saved:
+            pool.index_copy_(0, index, rows)
 
     def _generations(self) -> tuple:
         from .. import ops
@@ -423,8 +438,11 @@ class Engine:
             self.graph_replays += 1
             return held[1]
         # first time: an eager run settles the sizes of every work buffer (it writes the same
-        # keys and values the replay will write again), then capture and replay
+        # keys and values the replay will write again), then capture and replay.  State of
+        # fixed size is not written again but moved on: it is put back before the replay.
+        saved = self._save_states(ctx.slots)
         logits = self.model.forward(ctx, self.views)
+        self._restore_states(ctx.slots, saved)
         if held is not None or any(g[2] != self._generations() for g in self._graphs.values()):
             # a work buffer has moved: every graph that holds its old address is dead
             self._graphs = {k: g for k, g in self._graphs.items()

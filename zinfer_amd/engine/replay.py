@@ -36,7 +36,7 @@ from .batch import StepEntry
 from .engine import Engine
 
 PAGE_SIZE = 16
-MAX_LIVE_REQUESTS = 16
+MAX_LIVE_REQUESTS = 4
 
 
 def pages_for(max_tokens: int, page_size: int) -> int:

@@ -23,11 +23,18 @@ class DecoderModel:
                        for i, b in enumerate(spec.layers)]
         self.final_norm = build_part("norm", spec.final_norm, ctx, spec.final_norm_prefix)
         self.graph_safe = self.final_norm.graph_safe and all(b.graph_safe for b in self.blocks)
+        # (inspection) called with (schedule position, the stream) behind every run of a block
+        self.layer_probe = None
         # embedding, row gather and head are the model's own launches
         self.kernel_modules = tuple(sorted(
             {"elementwise", "gemm"} | ({"norms"} if spec.position_table_name is not None else set())
             | set(self.final_norm.kernel_modules)
             | {m for b in self.blocks for m in b.kernel_modules}))
+        if spec.position_table_name is not None and spec.sinusoidal_positions is not None:
+            raise ConfigError("a learned position table or computed position vectors, not both")
+        if any(e.reentry for e in spec.schedule) and spec.reentry_name is None:
+            raise ConfigError("a run of the schedule re-enters the embedding's output, but the "
+                              "model names no matrix for it")
         for pos, e in enumerate(spec.schedule):
             if not (0 <= e.layer < len(self.blocks)):
                 raise ConfigError(f"schedule[{pos}] names layer {e.layer} of {len(self.blocks)}")
@@ -46,6 +53,9 @@ class DecoderModel:
         d: Dict[str, TensorDecl] = {s.embed_name: TensorDecl((s.vocab_size, s.hidden_size))}
         if s.position_table_name is not None:
             d[s.position_table_name] = TensorDecl((s.max_positions, s.hidden_size))
+        if s.reentry_name is not None:
+            d[s.reentry_name] = TensorDecl((s.hidden_size, 2 * s.hidden_size),
+                                           optional=not any(e.reentry for e in s.schedule))
         for b in self.blocks:
             d.update(b.declare())
         d.update(self.final_norm.declare())
@@ -62,6 +72,16 @@ class DecoderModel:
             if table.dtype != tensors[s.embed_name].dtype:
                 table = table.to(tensors[s.embed_name].dtype)
             self.position_table = place_matrix(table, self.ctx)
+        self.position_freq = None
+        if s.sinusoidal_positions is not None:
+            # f_i = base^(-2i / width), formed in 64-bit once and kept as 32-bit numbers
+            i = torch.arange((s.hidden_size + 1) // 2, dtype=torch.float64)
+            base = torch.tensor(float(s.sinusoidal_positions.base), dtype=torch.float64)
+            self.position_freq = torch.pow(base, -2.0 * i / s.hidden_size) \
+                .to(torch.float32).to(self.ctx.device)
+        self.reentry = None
+        if s.reentry_name is not None and s.reentry_name in tensors:
+            self.reentry = Linear(place_matrix(tensors[s.reentry_name], self.ctx))
         for b in self.blocks:
             b.bind(tensors)
         self.final_norm.bind(tensors)
@@ -103,10 +123,24 @@ class DecoderModel:
         if self.position_table is not None:
             ops.embed_position(self.embedding, step.token_ids, self.position_table,
                                step.positions, x, float(s.embedding_multiplier))
+        elif self.position_freq is not None:
+            ops.embed_sinusoid(self.embedding, step.token_ids, step.positions,
+                               self.position_freq, x, float(s.embedding_multiplier))
         else:
             ops.embed(self.embedding, step.token_ids, x, float(s.embedding_multiplier))
+        x0 = None
+        if self.reentry is not None:
+            # the stream as the embedding left it, for the runs that re-enter it
+            x0 = step.scratch("embedding_out", (T, s.hidden_size), torch.float32)
+            x0.copy_(x)
         step.norm_ready = None
         for pos, e in enumerate(s.schedule):
+            if e.reentry:
+                # x = W [x ; x0]: both streams side by side in the products' type, one product
+                both = step.scratch("reentry_rows", (T, 2 * s.hidden_size), self.ctx.act_dtype)
+                ops.concat_rows(x, x0, both)
+                self.reentry.forward(both, x)
+                step.norm_ready = None
             # the norm that reads the stream after this block: the next block's first, or the
             # final norm when every row goes to the head as it lies
             if pos + 1 < len(s.schedule):
@@ -114,8 +148,12 @@ class DecoderModel:
             else:
                 after = self.final_norm if self.final_norm.defers and step.wants_all_rows \
                     else None
+            if pos + 1 < len(s.schedule) and s.schedule[pos + 1].reentry:
+                after = None            # the stream is replaced before the next block reads it
             step.norm_after_block = after
             self.blocks[e.layer].forward(x, step, caches[pos])
+            if self.layer_probe is not None:
+                self.layer_probe(pos, x)
         left, step.norm_ready, step.norm_after_block = step.norm_ready, None, None
         n_rows = step.n_want
         logits = step.scratch("logits", (n_rows, s.vocab_size), torch.float32)

@@ -144,6 +144,42 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: floa
                         ctypes.c_float(scale), _stream()), "embed")
 
 
+@_launches("other")
+def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+                   freq: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t, :] = table[ids[t], :] * scale plus a position vector formed where it is used:
+    entry 2i gets sin(p * freq[i]), entry 2i + 1 cos(p * freq[i]), p = positions[t]; the angle
+    is the 32-bit product.  ``freq`` float32 [ceil(H / 2)]."""
+    _need_gpu(table, ids, positions, freq, out)
+    _i32(ids, "ids")
+    _i32(positions, "positions")
+    T, H = out.shape
+    if table.shape[1] != H or ids.shape[0] != T or positions.shape[0] != T \
+            or out.dtype != torch.float32 or freq.dtype != torch.float32 \
+            or freq.shape != ((H + 1) // 2,):
+        raise KernelUnavailable(f"embed_sinusoid: table {tuple(table.shape)}, out "
+                                f"{tuple(out.shape)} {out.dtype}, freq {tuple(freq.shape)} "
+                                f"{freq.dtype}")
+    lib = build.load("elementwise")
+    _check(lib.zf_embed_sinusoid(_ptr(table), _dt(table), _ptr(ids), _ptr(positions), _ptr(freq),
+                                 _ptr(out), T, H, ctypes.c_float(scale), _stream()),
+           "embed_sinusoid")
+
+
+@_launches("other")
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = [a[t] | b[t]] for two float32 matrices [T, H], in ``out``'s type [T, 2 H]."""
+    _need_gpu(a, b, out)
+    T, H = a.shape
+    if b.shape != a.shape or out.shape != (T, 2 * H) or a.dtype != torch.float32 \
+            or b.dtype != torch.float32:
+        raise KernelUnavailable(f"concat_rows: float32 {tuple(a.shape)} and {tuple(b.shape)} "
+                                f"into {tuple(out.shape)}")
+    lib = build.load("elementwise")
+    _check(lib.zf_concat_rows(_ptr(a), _ptr(b), _ptr(out), _dt(out), T, H, _stream()),
+           "concat_rows")
+
+
 @_launches("head_sampling")
 def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> None:
     """In place on float32: x = x * scale, then with cap > 0: x = cap * tanh(x / cap)."""
@@ -1690,35 +1726,55 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
 MOE_MAX_EXPERTS = 1024
 
 
+ROUTER_SCORINGS = {"softmax": 0, "sigmoid": 1}
+
+
 @_launches("other")
 def moe_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor],
-              ids: torch.Tensor, weights: torch.Tensor) -> None:
+              ids: torch.Tensor, weights: torch.Tensor, scoring: str = "softmax",
+              correction: Optional[torch.Tensor] = None,
+              groups: Optional[Tuple[int, int]] = None) -> None:
     """Per row of ``h`` [T, W]: z = router h + bias in 32-bit (router float32 [E, W]); ``ids``
-    [T, top] int32 receives the ``top`` largest (the lower index wins a tie), ``weights``
-    [T, top] float32 the soft-max over those alone."""
-    _need_gpu(h, router, bias, ids, weights)
+    [T, top] int32 receives the ``top`` chosen experts (the lower index wins a tie).
+    ``scoring`` "softmax": the largest z are chosen and ``weights`` [T, top] float32 is the
+    soft-max over those alone.  "sigmoid": s = sigmoid(z); the choice goes by s + ``correction``
+    (float32 [E], or none); with ``groups`` = (count, keep) the experts form ``count`` equal
+    groups of neighbours, a group is marked by its two largest choice scores added, and only
+    experts of the ``keep`` best groups can be chosen; the weights are the chosen s over their
+    sum (+ 1e-20)."""
+    _need_gpu(h, router, bias, ids, weights, correction)
     _i32(ids, "ids")
     T, W = h.shape
     E = router.shape[0]
     top = ids.shape[1] if ids.dim() == 2 else 0
+    count, keep = groups if groups is not None else (0, 0)
     if router.dtype != torch.float32 or router.shape != (E, W) or ids.shape != (T, top) \
             or weights.shape != (T, top) or weights.dtype != torch.float32 \
-            or not 0 < top <= E <= MOE_MAX_EXPERTS \
-            or (bias is not None and (bias.dtype != torch.float32 or bias.shape != (E,))):
+            or not 0 < top <= E <= MOE_MAX_EXPERTS or scoring not in ROUTER_SCORINGS \
+            or (bias is not None and (bias.dtype != torch.float32 or bias.shape != (E,))) \
+            or (correction is not None and (correction.dtype != torch.float32
+                                            or correction.shape != (E,))) \
+            or (scoring == "softmax" and (correction is not None or groups is not None)) \
+            or (groups is not None and not (0 < keep <= count <= E and E % count == 0
+                                            and top <= keep * (E // count))):
         raise KernelUnavailable(f"moe_route: h {tuple(h.shape)}, router {tuple(router.shape)} "
                                 f"{router.dtype}, ids {tuple(ids.shape)}, at most "
-                                f"{MOE_MAX_EXPERTS} experts")
+                                f"{MOE_MAX_EXPERTS} experts, scoring {scoring!r}, groups {groups}")
     lib = build.load("moe")
     _check(lib.zf_moe_route(_ptr(h), _dt(h), _ptr(router), _ptr(bias), _ptr(ids), _ptr(weights),
-                            T, W, E, top, _stream()), "moe_route")
+                            T, W, E, top, ROUTER_SCORINGS[scoring], _ptr(correction), int(count),
+                            int(keep), _stream()), "moe_route")
 
 
 @_launches("products")
 def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, ids: Optional[torch.Tensor],
-                y: torch.Tensor, limit: float, alpha: float, shift: float) -> None:
+                y: torch.Tensor, limit: float, alpha: float, shift: float,
+                act: Optional[str] = None) -> None:
     """y[t, s, :] = act(expert ids[t, s] of ``gate_up`` [E, 2 ff, W] applied to h[t]) with
     g = min(gate, limit), u = clamp(up, -limit, limit) (no clamp if limit <= 0) and
-    act = g * sigmoid(alpha g) * (u + shift).  ``ids`` None: expert 0 for every token."""
+    act = g * sigmoid(alpha g) * (u + shift).  With ``act`` (one of ``ACTIVATIONS``) the experts
+    have no gate: ``gate_up`` is [E, ff, W] and y = act(up h).  ``ids`` None: expert 0 for every
+    token."""
     _need_gpu(h, gate_up, ids, y)
     T, W = h.shape
     if y.dim() != 3 or gate_up.dim() != 3:
@@ -1726,15 +1782,20 @@ def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, ids: Optional[torch.Tens
     slots, ff = y.shape[1], y.shape[2]
     if ids is not None:
         _i32(ids, "ids")
-    if y.shape[0] != T or gate_up.shape[1:] != (2 * ff, W) or gate_up.dtype != h.dtype \
+    rows = ff if act is not None else 2 * ff
+    if y.shape[0] != T or gate_up.shape[1:] != (rows, W) or gate_up.dtype != h.dtype \
             or y.dtype != h.dtype or (ids is not None and ids.shape != (T, slots)) \
-            or (ids is None and gate_up.shape[0] != 1) or W > 16384:
+            or (ids is None and gate_up.shape[0] != 1) or W > 16384 \
+            or (act is not None and act not in ACTIVATIONS):
         raise KernelUnavailable(f"moe_gate_up: h {tuple(h.shape)} {h.dtype}, gate_up "
-                                f"{tuple(gate_up.shape)} {gate_up.dtype}, y {tuple(y.shape)}")
+                                f"{tuple(gate_up.shape)} {gate_up.dtype}, y {tuple(y.shape)}, "
+                                f"activation {act!r}")
     lib = build.load("moe")
     _check(lib.zf_moe_gate_up(_ptr(h), _ptr(gate_up), _dt(h), _ptr(ids), _ptr(y), T, W, ff,
                               slots, ctypes.c_float(limit), ctypes.c_float(alpha),
-                              ctypes.c_float(shift), _stream()), "moe_gate_up")
+                              ctypes.c_float(shift), 0 if act is not None else 1,
+                              ACTIVATIONS[act] if act is not None else 0, _stream()),
+           "moe_gate_up")
 
 
 @_launches("products")
@@ -1780,45 +1841,50 @@ MOE_TILE_ROWS = 128           # MOE_TILE_ROWS in moe.hip
 MOE_STREAM_MAX_TOKENS = 16    # up to here every (token, expert) streams its own matrices
 
 
-def moe_grouped_covers(h: torch.Tensor, gate_up: torch.Tensor) -> bool:
+def moe_grouped_covers(h: torch.Tensor, gate_up: torch.Tensor, act: Optional[str] = None) -> bool:
     """Whether the MFMA kernels over tokens sorted by expert take these operands: bfloat16,
     both reduction lengths multiples of 8."""
+    ff = gate_up.shape[1] if act is not None else gate_up.shape[1] // 2
     return h.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 \
-        and gate_up.shape[2] % 8 == 0 and (gate_up.shape[1] // 2) % 8 == 0
+        and gate_up.shape[2] % 8 == 0 and ff % 8 == 0
 
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
                 weights: torch.Tensor, y: torch.Tensor, out: torch.Tensor, limit: float,
-                alpha: float, shift: float, add: bool = False) -> None:
+                alpha: float, shift: float, add: bool = False,
+                act: Optional[str] = None) -> None:
     """out[t] (=, +=) sum over s of weights[t, s] * expert ids[t, s] applied to h[t]
     (``moe_gate_up`` then ``moe_down``), with ``y`` [T, top, ff] as work space.  A few tokens
     stream each chosen expert's matrices (one workgroup row per token and slot); more tokens,
     in bfloat16, are sorted by expert and run through MFMA tiles of ``MOE_TILE_ROWS`` pairs
     (``moe_sort``, ``moe_grouped`` twice, ``moe_combine``).  Either way a token's result
-    depends on that token alone."""
+    depends on that token alone.  ``act``: experts without a gate (see ``moe_gate_up``)."""
     T, W = h.shape
-    if T > MOE_STREAM_MAX_TOKENS and moe_grouped_covers(h, gate_up):
-        moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add)
+    if T > MOE_STREAM_MAX_TOKENS and moe_grouped_covers(h, gate_up, act):
+        moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add, act)
         return
-    moe_gate_up(h, gate_up, ids, y, limit, alpha, shift)
+    moe_gate_up(h, gate_up, ids, y, limit, alpha, shift, act)
     moe_down(y, down, ids, weights, out, add=add)
 
 
 @_launches("products")
-def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add=False) -> None:
+def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add=False,
+                act: Optional[str] = None) -> None:
     """The many-token form of ``moe_experts`` (bfloat16; see there)."""
     _need_gpu(h, gate_up, down, ids, weights, y, out)
     _i32(ids, "ids")
     T, W = h.shape
-    E, ff2, _ = gate_up.shape
-    ff = ff2 // 2
+    E, rows, _ = gate_up.shape
+    ff = rows if act is not None else rows // 2
     top = ids.shape[1]
-    if not moe_grouped_covers(h, gate_up) or down.dtype != torch.bfloat16 \
-            or gate_up.shape != (E, 2 * ff, W) or down.shape != (E, W, ff) \
+    if not moe_grouped_covers(h, gate_up, act) or down.dtype != torch.bfloat16 \
+            or gate_up.shape != (E, ff if act is not None else 2 * ff, W) \
+            or down.shape != (E, W, ff) \
             or ids.shape != (T, top) or weights.shape != (T, top) \
             or weights.dtype != torch.float32 or y.dtype != torch.bfloat16 \
             or y.numel() != T * top * ff or not y.is_contiguous() \
-            or out.shape != (T, W) or out.dtype != torch.float32 or not 0 < E <= MOE_MAX_EXPERTS:
+            or out.shape != (T, W) or out.dtype != torch.float32 or not 0 < E <= MOE_MAX_EXPERTS \
+            or (act is not None and act not in ACTIVATIONS):
         raise KernelUnavailable(f"moe_grouped: h {tuple(h.shape)} {h.dtype}, gate_up "
                                 f"{tuple(gate_up.shape)}, down {tuple(down.shape)}, ids "
                                 f"{tuple(ids.shape)}, y {tuple(y.shape)} {y.dtype}")
@@ -1837,12 +1903,15 @@ def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add
     _check(lib.zf_moe_sort(_ptr(ids), P, E, _ptr(sorted_), _ptr(place), _ptr(tile_expert),
                            _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles), st), "moe_sort")
     lim, al, sh = ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift)
+    kind = ACTIVATIONS[act] if act is not None else 0
     _check(lib.zf_moe_grouped(_ptr(h), ctypes.c_longlong(W), _ptr(sorted_), top, _ptr(gate_up),
                               _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles),
-                              _ptr(y), max_tiles, ff, W, 1, lim, al, sh, st), "moe_grouped (gate, up)")
+                              _ptr(y), max_tiles, ff, W, 2 if act is not None else 1, lim, al, sh,
+                              kind, st), "moe_grouped (gate, up)")
     _check(lib.zf_moe_grouped(_ptr(y), ctypes.c_longlong(ff), _ptr(sorted_), top, _ptr(down),
                               _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles),
-                              _ptr(o), max_tiles, W, ff, 0, lim, al, sh, st), "moe_grouped (down)")
+                              _ptr(o), max_tiles, W, ff, 0, lim, al, sh, 0, st),
+           "moe_grouped (down)")
     _check(lib.zf_moe_combine(_ptr(o), _ptr(place), _ptr(weights), _ptr(out), T, W, top,
                               1 if add else 0, st), "moe_combine")
 
@@ -1886,13 +1955,14 @@ def sample_topk(logits: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -
 
 
 # ------------------------------------------------------------------------- an activation alone
-ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu2": 3, "tanh": 4}
 
 
 @_launches("norm_rope_write")
 def activation(x: torch.Tensor, out: torch.Tensor, kind: str) -> None:
     """out = act(x) element by element, in 32-bit on values of either storage type: "gelu"
-    (the exact form with erf), "gelu_tanh", "silu".  ``out`` may be ``x``."""
+    (the exact form with erf), "gelu_tanh", "silu", "relu2" (max(x, 0)^2), "tanh".  ``out``
+    may be ``x``."""
     _need_gpu(x, out)
     if x.shape != out.shape or x.dtype != out.dtype or kind not in ACTIVATIONS:
         raise KernelUnavailable(f"activation: {tuple(x.shape)} {x.dtype} -> {tuple(out.shape)} "
@@ -2139,7 +2209,7 @@ def head_products(a: torch.Tensor, a_off: int, a_hd: int, w: torch.Tensor,
 # (key width, value width) the MFMA kernels are built for: values of their own, and the keys'
 # leading columns as values
 MASKED_MFMA_SHAPES = {False: ((64, 64), (96, 96), (128, 128)),
-                      True: ((96, 64), (160, 128), (192, 128))}
+                      True: ((64, 64), (96, 96), (128, 128), (96, 64), (160, 128), (192, 128))}
 MASKED_MFMA_ROWS = 128           # (position, head) pairs a workgroup takes
 MASKED_ROWS_WAVES = 2048         # a prompt portion's keys are cut in parts until this many waves run
 MASKED_ROWS_MAX_PARTS = 4
@@ -2236,3 +2306,146 @@ def masked_attention_mfma(q, gate, gate_mode, k_pool, v_pool, sink, block_table,
         int(window), int(chunk), T, n_seqs, n_tiles, n_heads, n_kv_heads, key_width, value_width,
         page_size, max_pages, 1 if decode else 0, parts, wave_keys, _stream())
     _check(code, "masked_attention_mfma")
+
+
+# ------------------------------------------------------------------------- mixers with a state of fixed size
+RECURRENCE_CHANNELS = 8          # REC_R in recurrent.hip: key channels a thread holds
+RECURRENCE_MAX_KEY_DIM = 256
+RECURRENCE_MAX_THREADS = 256
+RECURRENCE_WORKGROUPS = 512      # value columns are dealt over workgroups until about this many run
+DECAY_RULES = {"sigmoid_root": 0, "double_exp": 1}
+
+
+def recurrence_state_size(n_heads: int, key_dim: int, value_dim: int) -> int:
+    """32-bit numbers a request's state takes in ``decay_recurrence``: [head][value column]
+    [channels padded to a multiple of ``RECURRENCE_CHANNELS``]."""
+    padded = (key_dim + RECURRENCE_CHANNELS - 1) // RECURRENCE_CHANNELS * RECURRENCE_CHANNELS
+    return n_heads * value_dim * padded
+
+
+def recurrence_state_matrix(state: torch.Tensor, n_heads: int, key_dim: int,
+                            value_dim: int) -> torch.Tensor:
+    """The matrices S [.., head, key channel, value column] of states laid out as the kernel
+    keeps them (tests and inspection)."""
+    padded = recurrence_state_size(n_heads, key_dim, value_dim) // (n_heads * value_dim)
+    s = state[..., :n_heads * value_dim * padded]
+    s = s.reshape(s.shape[:-1] + (n_heads, value_dim, padded))
+    return s[..., :key_dim].transpose(-1, -2)
+
+
+@_launches("norm_rope_write")
+def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, state_offset: int,
+                    state_slots: torch.Tensor, seq_index: torch.Tensor, q_start: torch.Tensor,
+                    out: torch.Tensor) -> None:
+    """out[m, t] = h[t] + (h[t - 1] - h[t]) * mu[m] for the rows ``h`` [T, W] of a step
+    (``mu`` float32 [n, W], ``out`` [n, T, W] in the rows' type).  The row before a sequence's
+    first row of this step is the request's state: elements [state_offset, state_offset + W)
+    of row state_slots[s] of ``state`` (float32 [slots, size]), which afterwards hold the
+    sequence's last row of this step."""
+    _need_gpu(h, mu, state, state_slots, seq_index, q_start, out)
+    for t, name in ((state_slots, "state_slots"), (seq_index, "seq_index"), (q_start, "q_start")):
+        _i32(t, name)
+    T, W = h.shape
+    n = mu.shape[0]
+    if mu.dtype != torch.float32 or mu.shape != (n, W) or out.shape != (n, T, W) \
+            or out.dtype != h.dtype or state.dtype != torch.float32 or state.dim() != 2 \
+            or not 0 <= state_offset <= state.shape[1] - W or seq_index.shape[0] != T \
+            or q_start.shape[0] != state_slots.shape[0] + 1:
+        raise KernelUnavailable(f"token_shift_mix: h {tuple(h.shape)}, mu {tuple(mu.shape)} "
+                                f"{mu.dtype}, out {tuple(out.shape)}, state {tuple(state.shape)} "
+                                f"{state.dtype} from {state_offset}")
+    lib = build.load("recurrent")
+    base = _vp(state.data_ptr() + 4 * int(state_offset))
+    _check(lib.zf_token_shift_mix(_ptr(h), _dt(h), _ptr(mu), base,
+                                  ctypes.c_longlong(state.shape[1]), _ptr(state_slots),
+                                  _ptr(seq_index), _ptr(q_start), _ptr(out), T, W, n, _stream()),
+           "token_shift_mix")
+
+
+def _recurrence_columns(n_seqs: int, n_heads: int, key_dim: int, value_dim: int) -> int:
+    """Value columns a workgroup of ``decay_recurrence`` takes: as many as its threads hold,
+    fewer where that leaves the chip idle.  The results do not depend on it."""
+    groups = (key_dim + RECURRENCE_CHANNELS - 1) // RECURRENCE_CHANNELS
+    most = max(1, min(value_dim, RECURRENCE_MAX_THREADS // groups))
+    vb = most
+    while vb > 8 and n_seqs * n_heads * ((value_dim + vb - 1) // vb) < RECURRENCE_WORKGROUPS:
+        vb = (vb + 1) // 2
+    return vb
+
+
+@_launches("attention")
+def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
+                     z_bias: torch.Tensor, bonus: Optional[torch.Tensor], state: torch.Tensor,
+                     state_slots: torch.Tensor, q_start: torch.Tensor, out: torch.Tensor,
+                     n_heads: int, key_dim: int, value_dim: int, rule: str, tau: float = 1.0,
+                     q_scale: float = 1.0, columns: Optional[int] = None) -> None:
+    """The recurrence S_t = diag(a_t) S_(t-1) + k_t v_t^T a head, token by token in 32-bit, over
+    the rows of a step: ``q``, ``k`` [T, H * d] and ``v`` [T, H * dv] (contiguous rows, any row
+    stride), ``z`` float32 [T, H * d] with a_t = sigmoid(z_t + z_bias)^(1 / tau) (``rule``
+    "sigmoid_root") or exp(-exp(z_t + z_bias)) ("double_exp").  Without ``bonus`` the output is
+    o_t = S_t^T (q_t * q_scale); with ``bonus`` u (float32 [H * d]) it is
+    o_t = (S_(t-1) + diag(u) k_t v_t^T)^T (q_t * q_scale).  ``out`` float32 [T, H * dv].
+    Sequence s owns the rows q_start[s] .. q_start[s + 1] - 1; its state (row state_slots[s] of
+    ``state``, float32 [slots, >= ``recurrence_state_size``]) is read before its first row and
+    written behind its last.  A row's result depends on the state and the rows of its own
+    sequence alone, and not on how the sequence was cut into steps."""
+    _need_gpu(z, z_bias, bonus, state, state_slots, q_start, out)
+    for t in (q, k, v):
+        if not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    _i32(state_slots, "state_slots")
+    _i32(q_start, "q_start")
+    T = q.shape[0]
+    H, d, dv = int(n_heads), int(key_dim), int(value_dim)
+    n_seqs = state_slots.shape[0]
+    need = recurrence_state_size(H, d, dv)
+    if rule not in DECAY_RULES or not 0 < d <= RECURRENCE_MAX_KEY_DIM or dv < 1 or H < 1 \
+            or q.shape[1] < H * d or k.shape[1] < H * d or v.shape[1] < H * dv \
+            or k.shape[0] != T or v.shape[0] != T or k.dtype != q.dtype or v.dtype != q.dtype \
+            or z.shape != (T, H * d) or z.dtype != torch.float32 \
+            or z_bias.shape != (H * d,) or z_bias.dtype != torch.float32 \
+            or (bonus is not None and (bonus.shape != (H * d,) or bonus.dtype != torch.float32)) \
+            or out.shape != (T, H * dv) or out.dtype != torch.float32 \
+            or state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < need \
+            or q_start.shape[0] != n_seqs + 1 or not tau > 0.0:
+        raise KernelUnavailable(f"decay_recurrence: q {tuple(q.shape)}, k {tuple(k.shape)}, v "
+                                f"{tuple(v.shape)} {q.dtype}, z {tuple(z.shape)} {z.dtype}, out "
+                                f"{tuple(out.shape)} {out.dtype}, state {tuple(state.shape)} for "
+                                f"{H} heads of {d} x {dv} (key size up to "
+                                f"{RECURRENCE_MAX_KEY_DIM}), rule {rule!r}")
+    vb = int(columns) if columns is not None else _recurrence_columns(n_seqs, H, d, dv)
+    lib = build.load("recurrent")
+    code = lib.zf_decay_recurrence(
+        _ptr(q), ctypes.c_longlong(_columns(q, "decay_recurrence: q")), _ptr(k),
+        ctypes.c_longlong(_columns(k, "decay_recurrence: k")), _ptr(v),
+        ctypes.c_longlong(_columns(v, "decay_recurrence: v")), _dt(q), _ptr(z), _ptr(z_bias),
+        _ptr(bonus), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(state_slots),
+        _ptr(q_start), _ptr(out), n_seqs, H, d, dv, vb, DECAY_RULES[rule],
+        ctypes.c_float(1.0 / tau), ctypes.c_float(q_scale), _stream())
+    _check(code, "decay_recurrence")
+
+
+@_launches("norm_rope_write")
+def head_norm_gate(o: torch.Tensor, gain: torch.Tensor, gate: torch.Tensor, out: torch.Tensor,
+                   n_heads: int, eps: float) -> None:
+    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * gain * silu(gate[t, h, :]):
+    ``o`` float32 [T, H * dv]; ``gain`` float32 [dv] (one for all heads) or [H * dv]; ``gate``
+    (contiguous rows, any row stride) and ``out`` [T, H * dv] in the products' type."""
+    _need_gpu(o, gain, out)
+    if not gate.is_cuda:
+        raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    T, width = o.shape
+    H = int(n_heads)
+    dv = width // H if H > 0 else 0
+    if H < 1 or dv * H != width or o.dtype != torch.float32 or gain.dtype != torch.float32 \
+            or gain.shape not in ((dv,), (width,)) or gate.shape != (T, width) \
+            or out.shape != (T, width) or gate.dtype != out.dtype:
+        raise KernelUnavailable(f"head_norm_gate: o {tuple(o.shape)} {o.dtype}, gain "
+                                f"{tuple(gain.shape)}, gate {tuple(gate.shape)} {gate.dtype}, out "
+                                f"{tuple(out.shape)} {out.dtype}, {H} heads")
+    lib = build.load("recurrent")
+    per_head = 1 if gain.shape == (width,) and H > 1 else 0
+    _check(lib.zf_head_norm_gate(_ptr(o), _ptr(gain), per_head, _ptr(gate),
+                                 ctypes.c_longlong(_columns(gate, "head_norm_gate: gate")),
+                                 _ptr(out), _dt(out), T, H, dv, ctypes.c_float(eps), _stream()),
+           "head_norm_gate")

@@ -10,6 +10,7 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from . import (gated_act, moe_grouped, norm_add_norm, tied_attention_mfma)
+from . import (concat_rows, decay_recurrence, embed_sinusoid, head_norm_gate, token_shift_mix)
 from . import (activation, head_products, masked_attention, masked_attention_mfma,
                norm_add_store, project_rows)
 from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
@@ -80,14 +81,15 @@ KERNELS: Dict[str, KernelEntry] = {
                                        "silent soft-max term and an output gate"),
     "tied_attention_mfma": KernelEntry(tied_attention_mfma, "sink_attention",
                                        "own: the same attention in MFMA tiles (bfloat16)"),
-    "moe_route": KernelEntry(moe_route, "moe", "own: router logits, top-k, soft-max of the chosen"),
+    "moe_route": KernelEntry(moe_route, "moe", "own: router logits, top-k, soft-max of the chosen "
+                             "or sigmoid scores chosen by corrected scores within the best groups"),
     "moe_gate_up": KernelEntry(moe_gate_up, "moe", "own: the chosen experts' gated activations"),
     "moe_down": KernelEntry(moe_down, "moe", "own: the chosen experts' outputs, weighted"),
     "moe_grouped": KernelEntry(moe_grouped, "moe", "own: the chosen experts over tokens sorted "
                                "by expert, MFMA tiles"),
     "gated_act": KernelEntry(gated_act, "moe", "own: the experts' activation alone"),
-    "activation": KernelEntry(activation, "elementwise", "own: gelu (erf or tanh form) or silu "
-                              "alone"),
+    "activation": KernelEntry(activation, "elementwise", "own: gelu (erf or tanh form), silu or "
+                              "squared relu alone"),
     "norm_add_store": KernelEntry(norm_add_store, "norms", "own: the norm behind a sublayer, the "
                                   "residual sum, and the sum in the products' type"),
     "project_rows": KernelEntry(project_rows, "masked_attention", "own: a projection's rows "
@@ -98,6 +100,16 @@ KERNELS: Dict[str, KernelEntry] = {
     "masked_attention_mfma": KernelEntry(masked_attention_mfma, "masked_attention",
                                          "own: the same attention in MFMA tiles (bfloat16)"),
     "head_products": KernelEntry(head_products, "masked_attention", "own: a matrix a head"),
+    "embed_sinusoid": KernelEntry(embed_sinusoid, "elementwise", "own: embedding plus a position "
+                                  "vector of sines and cosines"),
+    "concat_rows": KernelEntry(concat_rows, "elementwise", "own: two streams side by side for a "
+                               "product over both"),
+    "token_shift_mix": KernelEntry(token_shift_mix, "recurrent", "own: blends of a row with the "
+                                   "row before it, the last row kept as state"),
+    "decay_recurrence": KernelEntry(decay_recurrence, "recurrent", "own: a matrix a head, decayed "
+                                    "a key channel and grown by k v^T, token by token"),
+    "head_norm_gate": KernelEntry(head_norm_gate, "recurrent", "own: RMS norm a head, gain and "
+                                  "silu gate"),
     "mfma_loop": KernelEntry(mfma_loop, "gemm",
                              "own: MFMAs alone, the rate the tiled products are measured against"),
 }

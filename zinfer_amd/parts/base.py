@@ -39,10 +39,20 @@ from ..errors import ConfigError
 @dataclass(frozen=True)
 class TensorDecl:
     """A tensor a part binds.  ``init`` says how the random-weights mode draws it:
-    'normal' = N(0, 0.02), 'gain' = 1 + U(-0.1, 0.1)."""
-    shape: Tuple[int, ...]
+    'normal' = N(0, 0.02), 'gain' = 1 + U(-0.1, 0.1).  A dimension given as None is whatever the
+    file holds (the part reads it at ``bind``); ``free`` is its size when the tensor is drawn."""
+    shape: Tuple[Optional[int], ...]
     init: str = "normal"
     optional: bool = False
+    free: int = 16
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(
+            want is None or want == have for want, have in zip(self.shape, shape))
+
+    def drawn_shape(self) -> Tuple[int, ...]:
+        return tuple(self.free if d is None else d for d in self.shape)
 
 
 @dataclass(frozen=True)

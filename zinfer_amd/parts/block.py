@@ -4,7 +4,8 @@ from typing import Dict
 
 import torch
 
-from ..config.specs import PostNormBlockSpec, PreNormBlockSpec, SandwichNormBlockSpec
+from ..config.specs import (ParallelBlockSpec, PostNormBlockSpec, PreNormBlockSpec,
+                            SandwichNormBlockSpec)
 from .base import Block, TensorDecl, build_part, register_part
 
 
@@ -270,6 +271,59 @@ class PostNormBlock(Block):
         step.norm_ready = StreamRows(x, h) if h is not None else None
 
 
+class ParallelBlock(Block):
+    """x += mixer(norm1(x)) + feed_forward(norm2(x)): both norms read the stream before either
+    sublayer has added to it; the sublayers then add their outputs into the stream one after
+    the other, in 32-bit.  Without a feed-forward the block is its mixer's line."""
+
+    def __init__(self, spec: ParallelBlockSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx, prefix + spec.mixer_norm_prefix)
+        self.mixer = build_part("mixer", spec.mixer, ctx, prefix + spec.mixer_prefix)
+        self.parts = [self.mixer_norm, self.mixer]
+        self.ff_norm = self.feed_forward = None
+        if spec.feed_forward is not None:
+            self.ff_norm = build_part("norm", spec.ff_norm, ctx, prefix + spec.ff_norm_prefix)
+            self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
+                                           prefix + spec.ff_prefix)
+            self.parts += [self.ff_norm, self.feed_forward]
+        self.parts = tuple(self.parts)
+        self.graph_safe = all(p.graph_safe for p in self.parts)
+        self.kernel_modules = tuple(sorted({m for p in self.parts for m in p.kernel_modules}))
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        d: Dict[str, TensorDecl] = {}
+        for part in self.parts:
+            d.update(part.declare())
+        return d
+
+    def bind(self, tensors) -> None:
+        for part in self.parts:
+            part.bind(tensors)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def accept_cache(self, cache) -> None:
+        self.mixer.accept_cache(cache)
+
+    def hint_providers(self):
+        return [q for p in self.parts for q in p.hint_providers()]
+
+    def forward(self, x, step, cache) -> None:
+        step.norm_ready = step.norm_after = None
+        h1 = self.mixer_norm.forward(x, step.scratch("normed", x.shape, self.ctx.act_dtype))
+        h2 = None
+        if self.feed_forward is not None:
+            # (before the mixer adds into the stream: both sublayers read the same rows)
+            h2 = self.ff_norm.forward(x, step.scratch("normed_ff", x.shape, self.ctx.act_dtype))
+        self.mixer.forward(h1, x, step, cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(h2, x, step)
+        step.norm_ready = step.norm_after = None
+
+
+register_part("block", ParallelBlockSpec, ParallelBlock)
 register_part("block", PostNormBlockSpec, PostNormBlock)
 register_part("block", PreNormBlockSpec, PreNormBlock)
 register_part("block", SandwichNormBlockSpec, SandwichNormBlock)

@@ -138,8 +138,11 @@ class LatentAttention(Mixer):
     token, the attention runs with one kv head whose key row is [latent | rotated part] and
     whose value is the latent itself (the leading columns of the key row), and the head's
     value matrix is applied to the attention's output, with the gate in that product's
-    epilogue.  The cache holds kv_rank + rot_dim numbers a token whatever the number of
-    heads."""
+    epilogue (a gate an element) or in the attention's own (a gate a head: the value matrix
+    is linear, so the gate may stand on either side of it).  The cache holds kv_rank + rot_dim
+    numbers a token whatever the number of heads.  Without a query latent (``q_rank`` None) the
+    queries come out of the same product as the key latent; without a rotated part
+    (``rot_dim`` 0) the key row is the latent alone."""
     graph_safe = True
     stores_output = True
     kernel_modules = ("gemm", "masked_attention")
@@ -147,7 +150,8 @@ class LatentAttention(Mixer):
     def __init__(self, spec: LatentAttentionSpec, ctx, prefix):
         super().__init__(spec, ctx, prefix)
         s = spec
-        if min(s.n_heads, s.head_dim, s.rot_dim, s.value_dim, s.q_rank, s.kv_rank) < 1:
+        if min(s.n_heads, s.head_dim, s.value_dim, s.kv_rank) < 1 or s.rot_dim < 0 \
+                or (s.q_rank is not None and s.q_rank < 1):
             raise ConfigError("InvalidDimensions: heads, head sizes and ranks must be at least 1")
         if s.kv_rank > ops.MAX_HEAD_DIM:
             raise ConfigError(f"InvalidHeadDim: kv_rank={s.kv_rank}: the attention kernels take "
@@ -156,41 +160,53 @@ class LatentAttention(Mixer):
                                          and len(s.rotary.frequencies) == s.rot_dim // 2):
             raise ConfigError(f"the rotated part of a head ({s.rot_dim}) is rotated whole, not "
                               f"{s.rotary.dims} of it")
+        if s.element_gate and s.head_gate:
+            raise ConfigError("a gate an element or a gate a head, not both")
         _check_mask(s)
         self.q_head = s.head_dim + s.rot_dim
         self.key_width = s.kv_rank + s.rot_dim
+        self.gate_width = s.n_heads * s.value_dim if s.element_gate else \
+            (s.n_heads if s.head_gate else 0)
         self.freq = _frequencies(s.rotary, ctx)
 
     def declare(self) -> Dict[str, TensorDecl]:
         s, p = self.spec, self.prefix
-        d = {p + s.dq_name: TensorDecl((s.q_rank, s.hidden_size)),
-             p + s.dq_norm_name: TensorDecl((s.q_rank,), init="gain"),
-             p + s.uq_name: TensorDecl((s.n_heads * self.q_head, s.q_rank)),
-             p + s.dkv_name: TensorDecl((self.key_width, s.hidden_size)),
+        d = {p + s.dkv_name: TensorDecl((self.key_width, s.hidden_size)),
              p + s.dkv_norm_name: TensorDecl((s.kv_rank,), init="gain"),
              p + s.uk_name: TensorDecl((s.n_heads * s.head_dim, s.kv_rank)),
              p + s.uv_name: TensorDecl((s.n_heads * s.value_dim, s.kv_rank)),
              p + s.o_name: TensorDecl((s.hidden_size, s.n_heads * s.value_dim))}
-        if s.element_gate:
-            d[p + s.gate_name] = TensorDecl((s.n_heads * s.value_dim, s.hidden_size))
+        if s.q_rank is not None:
+            d[p + s.dq_name] = TensorDecl((s.q_rank, s.hidden_size))
+            d[p + s.dq_norm_name] = TensorDecl((s.q_rank,), init="gain")
+            d[p + s.uq_name] = TensorDecl((s.n_heads * self.q_head, s.q_rank))
+        else:
+            d[p + s.uq_name] = TensorDecl((s.n_heads * self.q_head, s.hidden_size))
+        if self.gate_width:
+            d[p + s.gate_name] = TensorDecl((self.gate_width, s.hidden_size))
         return d
 
     def bind(self, tensors) -> None:
         s, p = self.spec, self.prefix
-        rows = [tensors[p + s.dq_name], tensors[p + s.dkv_name]]
-        if s.element_gate:
+        # one product over the stacked matrices: [query latent or queries | key latent | gate]
+        first = tensors[p + s.dq_name] if s.q_rank is not None else tensors[p + s.uq_name]
+        rows = [first, tensors[p + s.dkv_name]]
+        if self.gate_width:
             rows.append(tensors[p + s.gate_name])
         if len({t.dtype for t in rows}) > 1:
             rows = [t.float() for t in rows]
+        self.first_width = first.shape[0]
         self.down = Linear(place_matrix(torch.cat(rows, dim=0), self.ctx))
-        self.uq = Linear(place_matrix(tensors[p + s.uq_name], self.ctx))
+        self.uq = self.dq_gain = None
+        if s.q_rank is not None:
+            self.uq = Linear(place_matrix(tensors[p + s.uq_name], self.ctx))
+            self.dq_gain = place_gain(tensors[p + s.dq_norm_name], self.ctx)
         self.o = Linear(place_matrix(tensors[p + s.o_name], self.ctx))
         # [H, kv_rank, head_dim]: the key matrix of a head, transposed, takes a query to the latent
         uk = tensors[p + s.uk_name].view(s.n_heads, s.head_dim, s.kv_rank).transpose(1, 2)
         self.uk_t = place_matrix(uk.contiguous(), self.ctx)
         self.uv = place_matrix(tensors[p + s.uv_name].view(s.n_heads, s.value_dim, s.kv_rank)
                                .contiguous(), self.ctx)
-        self.dq_gain = place_gain(tensors[p + s.dq_norm_name], self.ctx)
         self.dkv_gain = place_gain(tensors[p + s.dkv_norm_name], self.ctx)
 
     def cache_need(self):
@@ -211,37 +227,48 @@ class LatentAttention(Mixer):
         if hasattr(h, "materialize"):
             h = h.materialize()
         kv = step.kv_tables(cache.group)
-        KW, H = self.key_width, s.n_heads
+        KW, H, F = self.key_width, s.n_heads, self.first_width
         rot = dict(rot_dims=s.rot_dim, freq=self.freq, mag=s.rotary.magnitude) \
             if s.rotary is not None else {}
         down = step.scratch("latent_down", (T, self.down.out_features), act)
         self.down.forward(h, down)
-        cq = step.scratch("latent_cq", (T, s.q_rank), act)
-        segments = [ops.RowSegment(0, s.q_rank, cq, gain=self.dq_gain, eps=float(s.norm_eps))]
+        segments = []
+        if s.q_rank is not None:
+            cq = step.scratch("latent_cq", (T, s.q_rank), act)
+            segments.append(ops.RowSegment(0, s.q_rank, cq, gain=self.dq_gain,
+                                           eps=float(s.norm_eps)))
         if cache.writes:
-            segments.append(ops.RowSegment(s.q_rank, s.kv_rank, cache.k_pool, gain=self.dkv_gain,
+            segments.append(ops.RowSegment(F, s.kv_rank, cache.k_pool, gain=self.dkv_gain,
                                            eps=float(s.norm_eps), dst_hd=KW, pool_heads=1))
-            segments.append(ops.RowSegment(s.q_rank + s.kv_rank, s.rot_dim, cache.k_pool,
-                                           dst_off=s.kv_rank, dst_hd=KW, pool_heads=1, **rot))
-        ops.project_rows(down, step.positions, kv.slot_mapping if cache.writes else None,
-                         cache.page_size, segments)
-        q = step.scratch("latent_q", (T, H * self.q_head), act)
-        self.uq.forward(cq, q)
+            if s.rot_dim:
+                segments.append(ops.RowSegment(F + s.kv_rank, s.rot_dim, cache.k_pool,
+                                               dst_off=s.kv_rank, dst_hd=KW, pool_heads=1, **rot))
+        if segments:
+            ops.project_rows(down, step.positions, kv.slot_mapping if cache.writes else None,
+                             cache.page_size, segments)
+        if s.q_rank is not None:
+            q = step.scratch("latent_q", (T, H * self.q_head), act)
+            self.uq.forward(cq, q)
+        else:
+            q = down[:, :F]
         # the query on the latent's side: [U_h^T q_plain | rotated q_rot] a head
         qa = step.scratch("latent_qa", (T, H * KW), act)
         ops.head_products(q, 0, self.q_head, self.uk_t, None, qa, 0, KW)
-        ops.project_rows(q, step.positions, None, cache.page_size,
-                         [ops.RowSegment(0, H * self.q_head, qa, hd=self.q_head,
-                                         rot_off=s.head_dim, skip=s.head_dim, dst_off=s.kv_rank,
-                                         dst_hd=KW, **rot)])
+        if s.rot_dim:
+            ops.project_rows(q, step.positions, None, cache.page_size,
+                             [ops.RowSegment(0, H * self.q_head, qa, hd=self.q_head,
+                                             rot_off=s.head_dim, skip=s.head_dim,
+                                             dst_off=s.kv_rank, dst_hd=KW, **rot)])
+        gate = down[:, F + KW:] if self.gate_width else None
         mixed = step.scratch("latent_mixed", (T, H * s.kv_rank), act)
-        ops.attend_masked(qa, None, None, cache.k_pool, None, None, kv.block_table,
+        ops.attend_masked(qa, gate if s.head_gate else None, "head" if s.head_gate else None,
+                          cache.k_pool, None, None, kv.block_table,
                           step.q_start, step.ctx_len, step.seq_index, mixed, float(s.scale), 0.0,
                           int(s.window or 0), int(s.chunk or 0), H, 1, KW, s.kv_rank,
                           cache.page_size, step.max_q_len, step.max_ctx_len)
-        gate = down[:, s.q_rank + KW:] if s.element_gate else None
         attn = step.scratch("attn", (T, H * s.value_dim), act)
-        ops.head_products(mixed, 0, s.kv_rank, self.uv, gate, attn, 0, s.value_dim)
+        ops.head_products(mixed, 0, s.kv_rank, self.uv, gate if s.element_gate else None, attn, 0,
+                          s.value_dim)
         self.o.forward(attn, residual, accumulate=accumulate, step=step if accumulate else None)
 
 

@@ -5,7 +5,7 @@ from typing import Dict
 import torch
 
 from .. import ops
-from ..config.specs import MoeSpec
+from ..config.specs import MoeSpec, PlainExpertSpec
 from ..errors import ConfigError
 from .base import FeedForward, TensorDecl, register_part
 from .linear import Linear, place_gain, place_matrix
@@ -16,8 +16,11 @@ class MoeFeedForward(FeedForward):
     the ``top_k`` largest choose a token's experts, the soft-max over the chosen logits alone
     weighs them; an expert is W_down act(W_gate h, W_up h) with the clamped, gated activation
     of ``GatedExpertSpec``; an optional shared expert runs for every token and is added with
-    weight 1.  The experts' matrices are stacked at load (gate rows above up rows, expert by
-    expert) so that the kernels find an expert by its number.  Every token's sum runs over its
+    weight 1; with ``scoring`` "sigmoid" the router is the one ``MoeSpec`` describes (sigmoid
+    scores, a correction that enters the choice only, groups of experts), and a
+    ``PlainExpertSpec`` is an expert without a gate, W_down act(W_up h).  The experts' matrices
+    are stacked at load (gate rows above up rows, expert by expert) so that the kernels find an
+    expert by its number.  Every token's sum runs over its
     chosen experts in the order the router ranked them, then the shared one."""
     graph_safe = True
     stores_output = True
@@ -28,6 +31,25 @@ class MoeFeedForward(FeedForward):
         if not 1 <= spec.top_k <= spec.n_experts <= ops.MOE_MAX_EXPERTS:
             raise ConfigError(f"a mixture of {spec.n_experts} experts with {spec.top_k} a token: "
                               f"1 <= top <= experts <= {ops.MOE_MAX_EXPERTS}")
+        self.plain = isinstance(spec.expert, PlainExpertSpec)
+        if self.plain and spec.expert.activation not in ops.ACTIVATIONS:
+            raise ConfigError(f"activation {spec.expert.activation!r}: known are "
+                              f"{sorted(ops.ACTIVATIONS)}")
+        if spec.scoring not in ops.ROUTER_SCORINGS:
+            raise ConfigError(f"router scoring {spec.scoring!r}: known are "
+                              f"{sorted(ops.ROUTER_SCORINGS)}")
+        if spec.scoring == "softmax" and (spec.correction_name is not None
+                                          or spec.groups is not None):
+            raise ConfigError("a correction of the choice and groups of experts belong to the "
+                              "sigmoid router")
+        if spec.groups is not None:
+            count, keep = spec.groups
+            if not (0 < keep <= count <= spec.n_experts and spec.n_experts % count == 0
+                    and spec.top_k <= keep * (spec.n_experts // count)):
+                raise ConfigError(f"{spec.n_experts} experts in {count} equal groups, {keep} "
+                                  f"kept, {spec.top_k} chosen do not fit together")
+        if self.plain and spec.shared is not None:
+            raise ConfigError("a shared expert is a gated one")
 
     def _expert_names(self, prefix: str):
         s = self.spec
@@ -38,6 +60,14 @@ class MoeFeedForward(FeedForward):
         d = {p + s.router_name: TensorDecl((s.n_experts, s.hidden_size))}
         if s.router_bias:
             d[p + s.router_bias_name] = TensorDecl((s.n_experts,))
+        if s.correction_name is not None:
+            d[p + s.correction_name] = TensorDecl((s.n_experts,))
+        if self.plain:
+            for e in range(s.n_experts):
+                prefix = p + s.expert_prefix.format(e)
+                d[prefix + s.up_name] = TensorDecl((s.expert.intermediate_size, s.hidden_size))
+                d[prefix + s.down_name] = TensorDecl((s.hidden_size, s.expert.intermediate_size))
+            return d
         groups = [(p + s.expert_prefix.format(e), s.expert) for e in range(s.n_experts)]
         if s.shared is not None:
             groups.append((p + s.shared_prefix, s.shared))
@@ -53,10 +83,15 @@ class MoeFeedForward(FeedForward):
         device in the compute dtype, built expert by expert."""
         gate_up, down = [], []
         for prefix in prefixes:
-            g, u, dn = (tensors[n] for n in self._expert_names(prefix))
-            if g.dtype != u.dtype:
-                g, u = g.float(), u.float()
-            gate_up.append(place_matrix(torch.cat([g, u], dim=0), self.ctx))
+            gn, un, dnn = self._expert_names(prefix)
+            u, dn = tensors[un], tensors[dnn]
+            if self.plain:                  # no gate: the up rows alone
+                gate_up.append(place_matrix(u, self.ctx))
+            else:
+                g = tensors[gn]
+                if g.dtype != u.dtype:
+                    g, u = g.float(), u.float()
+                gate_up.append(place_matrix(torch.cat([g, u], dim=0), self.ctx))
             down.append(place_matrix(dn, self.ctx))
         dtypes = {t.dtype for t in gate_up + down}
         if len(dtypes) > 1:
@@ -69,6 +104,8 @@ class MoeFeedForward(FeedForward):
         self.router = place_gain(tensors[p + s.router_name], self.ctx)
         self.router_bias = place_gain(tensors[p + s.router_bias_name], self.ctx) \
             if s.router_bias else None
+        self.correction = place_gain(tensors[p + s.correction_name], self.ctx) \
+            if s.correction_name is not None else None
         self.gate_up, self.down = self._stack(
             tensors, [p + s.expert_prefix.format(e) for e in range(s.n_experts)])
         if s.shared is not None:
@@ -86,11 +123,17 @@ class MoeFeedForward(FeedForward):
             raise ConfigError(f"the experts are held in {dtype}, the activations in {h.dtype}")
         ids = step.scratch("moe_ids", (T, s.top_k), torch.int32)
         share = step.scratch("moe_share", (T, s.top_k), torch.float32)
-        ops.moe_route(h, self.router, self.router_bias, ids, share)
+        ops.moe_route(h, self.router, self.router_bias, ids, share, scoring=s.scoring,
+                      correction=self.correction, groups=s.groups)
         ex = s.expert
         y = step.scratch("moe_act", (T, s.top_k, ex.intermediate_size), dtype)
-        ops.moe_experts(h, self.gate_up, self.down, ids, share, y, residual,
-                        float(ex.limit or 0.0), float(ex.alpha), float(ex.shift), add=accumulate)
+        if self.plain:
+            ops.moe_experts(h, self.gate_up, self.down, ids, share, y, residual, 0.0, 1.0, 0.0,
+                            add=accumulate, act=ex.activation)
+        else:
+            ops.moe_experts(h, self.gate_up, self.down, ids, share, y, residual,
+                            float(ex.limit or 0.0), float(ex.alpha), float(ex.shift),
+                            add=accumulate)
         if s.shared is not None:
             sh = s.shared
             gu = step.scratch("moe_shared_gate_up", (T, 2 * sh.intermediate_size), dtype)

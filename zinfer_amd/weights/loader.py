@@ -55,7 +55,7 @@ def load_tensors(model_dir: str, decls: Dict[str, TensorDecl]) -> Dict[str, torc
             if n not in where:
                 continue
             info = where[n].infos[n]
-            if tuple(info.shape) != tuple(d.shape):
+            if not d.fits(info.shape):
                 wrong.append(f"{n}: expected shape {list(d.shape)}, file has {list(info.shape)}")
             elif info.dtype not in _FLOAT + _INT:
                 wrong.append(f"{n}: dtype {info.dtype} is not readable")

@@ -37,15 +37,16 @@ def draw_tensor(name: str, decl: TensorDecl, seed: int, dtype: torch.dtype,
         raise ValueError(f"random weights are stored as float32 or bfloat16, not {dtype}")
     if decl.init not in counter_rng.KIND:
         raise ValueError(f"tensor {name!r}: unknown init {decl.init!r}")
+    shape = decl.drawn_shape()
     n = 1
-    for d in decl.shape:
+    for d in shape:
         n *= d
     key = counter_rng.tensor_key(seed, name)
     if _on_gpu(device):
         from .. import ops
         out = torch.empty((n,), dtype=dtype, device=device)
         ops.randinit(out, key, 0, decl.init, STD)
-        return out.view(*decl.shape)
+        return out.view(*shape)
     out = torch.empty((n,), dtype=dtype)
     for lo in range(0, n, _CHUNK):            # in pieces: a big matrix never exists in 64-bit
         m = min(_CHUNK, n - lo)
@@ -55,7 +56,7 @@ def draw_tensor(name: str, decl: TensorDecl, seed: int, dtype: torch.dtype,
             out[lo:lo + m] = torch.from_numpy(bits).view(torch.bfloat16)
         else:
             out[lo:lo + m] = torch.from_numpy(piece)
-    return out.view(*decl.shape)
+    return out.view(*shape)
 
 
 class DrawnTensors(Mapping):
