@@ -158,6 +158,11 @@ TESTED_AGAINST = {
     "masked_attention": "plain_lodenex.py:masked_softmax_values",
     "masked_attention_mfma": "plain_lodenex.py:masked_softmax_values",
     "head_products": "test_lodenex_kernels_gpu.py:test_head_products",
+    "embed_sinusoid": "plain_nupovik.py:position_vectors",
+    "concat_rows": "test_nupovik_kernels_gpu.py:test_concat_rows",
+    "token_shift_mix": "plain_nupovik.py:token_shift",
+    "decay_recurrence": "plain_nupovik.py:decayed_outer_recurrence",
+    "head_norm_gate": "test_nupovik_kernels_gpu.py:test_head_norm_gate",
 }
 
 
