@@ -451,6 +451,8 @@ def test_a_loud_latent_far_back(dt, decode, R):
     c[n - 1] = 0.0
     c[n - 1, 0, 0], c[n - 1, 0, 1] = 30.0, 5.0
     pg = Paged([n], 1, R, 0, ps, dt, 93, k=[c])
-    got = _attend(pg, q[:2].to(dt), [2], dt, H, R, 1.0, None)
+    q2 = torch.zeros((2, H, R))
+    q2[:, :, 0] = 1.0
+    got = _attend(pg, q2.to(dt), [2], dt, H, R, 1.0, None)
     assert float(got[0, :, 1].float().abs().max()) < 1.0
     assert float((got[1, :, 1].float() - 5.0).abs().max()) < 0.05
