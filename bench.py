@@ -23,9 +23,10 @@ intermediate 25600; 65.5 GB of weights): a 2048-token prefill, then decode at ba
 64 with every request's context just below 8192 tokens; the cache pool is sized for
 64 x 8192 tokens (137 GB).
 
-``--workload fezupel`` and ``--workload lodenex``: shapes of those two designs at layer sizes that
-resemble served models, each beside the dense Qwen3 decoder of equal size (prefill of 2048
-tokens, decode at batch 8), and their kernels alone beside the like kernels of that decoder.
+``--workload fezupel``, ``--workload lodenex`` and ``--workload nupovik``: shapes of those three
+designs at layer sizes that resemble served models, each beside the dense Qwen3 decoder of equal
+size (prefill of 2048 tokens, decode at batch 8), and their kernels alone beside the like
+kernels of that decoder.
 
 The reference publishes no numbers, so ``vs_baseline`` is null.
 """
@@ -1005,10 +1006,291 @@ def main_lodenex(args) -> int:
     return 0
 
 
+# --------------------------------------------------------------------------- Nupovik beside Qwen3
+# Layer sizes that resemble served models with recurrent mixers; every shape is run beside the
+# dense Qwen3 decoder of the same width, depth and vocabulary, with heads of 128, whose gated
+# feed-forward does the matrix work a token of the new design's feed-forwards (a mixture counts
+# the experts a token uses).
+def _np_moe(experts, top, ff, groups):
+    return {"kind": "moe", "expert": {"ff": ff},
+            "router": {"experts": experts, "top": top,
+                       "groups": {"count": groups[0], "keep": groups[1]}}}
+
+
+NUPOVIK_SHAPES = {
+    # recurrent layers alone: token-shift layers with heads of 64, gated linear attention with
+    # keys half as wide as the values
+    "recurrent": dict(width=2048, vocab=32768, loop=None, layers=[
+        ("wkv", dict(heads=32, dim=64), {"kind": "dense", "ff": 7168}),
+        ("gla", dict(heads=8, dim=128, vdim=256, tau=16.0), {"kind": "dense", "ff": 7168}),
+        ("wkv", dict(heads=32, dim=64), {"kind": "dense", "ff": 7168}),
+        ("gla", dict(heads=8, dim=128, vdim=256, tau=16.0), {"kind": "dense", "ff": 7168})]),
+    # all three mixers, a mixture of 32 experts in 8 groups, the first two layers run twice
+    "hybrid": dict(width=4096, vocab=32768, loop=dict(start=0, stop=2, times=2), layers=[
+        ("gla", dict(heads=16, dim=128, vdim=256, tau=16.0), {"kind": "dense", "ff": 12288}),
+        ("latent_attention", dict(heads=32, dim=128, vdim=128, kv_rank=128, scale=128 ** -0.5),
+         _np_moe(32, 4, 2048, (8, 4))),
+        ("wkv", dict(heads=64, dim=64), _np_moe(32, 4, 2048, (8, 4))),
+        ("latent_attention", dict(heads=32, dim=128, vdim=128, kv_rank=128, scale=128 ** -0.5),
+         {"kind": "dense", "ff": 12288})]),
+}
+
+
+def nupovik_config(sh: dict) -> dict:
+    return {"architecture": "Nupovik", "vocab": sh["vocab"], "width": sh["width"],
+            "norm": {"eps": 1e-6}, "logit_scale": 1.0, "loop": sh["loop"],
+            "layers": [{"type": kind, "mixer": dict(mixer), "mlp": mlp}
+                       for kind, mixer, mlp in sh["layers"]]}
+
+
+def nupovik_runs(sh: dict) -> list:
+    """The layers in the order they run, a repeated one once a pass."""
+    n = len(sh["layers"])
+    if sh["loop"] is None:
+        return list(range(n))
+    a, b, times = sh["loop"]["start"], sh["loop"]["stop"], sh["loop"]["times"]
+    return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
+
+
+def nupovik_twin(sh: dict, max_positions: int) -> dict:
+    runs = nupovik_runs(sh)
+    used = [m["ff"] if m["kind"] == "dense" else m["router"]["top"] * m["expert"]["ff"]
+            for m in (sh["layers"][i][2] for i in runs)]
+    inter = int(sum(used) / len(used)) * 2 // 3 // 64 * 64
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+                num_hidden_layers=len(runs), hidden_size=sh["width"],
+                num_attention_heads=sh["width"] // 128, num_key_value_heads=8, head_dim=128,
+                intermediate_size=inter, vocab_size=sh["vocab"], rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=False,
+                max_position_embeddings=max_positions, torch_dtype="bfloat16")
+
+
+def nupovik_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float) -> dict:
+    """The new design's kernels alone beside the like kernels of the dense decoder, at ``T``
+    tokens of one sequence that holds ``ctx`` tokens (T = ctx: a prompt; T = 1 x 8 sequences: a
+    decode step).  Each has the fraction of its bound it reaches.  Matrix work: the MFMA loop's
+    rate (prompt) or the bytes that must be read against the measured read stream (decode).
+    The recurrence is 32-bit vector work, five operations a state element a token (prompt:
+    against the published 32-bit vector rate), or its state read and written once (decode)."""
+    import torch
+    import zinfer_amd.ops as ops
+    dev = "cuda:0"
+    W = sh["width"]
+    nH, nKV, hd = W // 128, 8, 128
+    bf = torch.bfloat16
+    decode = T == 1
+    n_seqs = 8 if decode else 1
+    rows = n_seqs * T
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev) * 0.05).to(bf)
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)
+    pages = (ctx + PAGE - 1) // PAGE
+    table = torch.arange(n_seqs * pages, dtype=torch.int32, device=dev).view(n_seqs, pages)
+    q_start = i32([i * T for i in range(n_seqs + 1)])
+    ctx_len = i32([ctx] * n_seqs)
+    seq_index = i32([i for i in range(n_seqs) for _ in range(T)])
+    state_slots = i32(list(range(n_seqs)))
+    out = {}
+
+    def row(name, t_new, work_new, rate_new, bound_new, t_old=None, work_old=None, rate_old=None,
+            bound_old=None):
+        r = {"nupovik_us": round(t_new * 1e6, 1),
+             "nupovik_frac_of_" + bound_new: round(work_new / t_new / rate_new, 4)}
+        if t_old is not None:
+            r.update({"qwen3_us": round(t_old * 1e6, 1),
+                      "qwen3_frac_of_" + bound_old: round(work_old / t_old / rate_old, 4)})
+        out[name] = r
+
+    mat_bound, mat_rate = ("read", read_bw) if decode else ("mfma", mfma_rate)
+    # ---- the dense decoder's attention at the twin's heads
+    q = rnd(rows, nH * hd)
+    k_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    v_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    o = torch.empty((rows, nH * hd), dtype=bf, device=dev)
+    t_att = _timed_graph(lambda: ops.paged_attention(q, k_pool, v_pool, table, q_start, ctx_len,
+                                                     seq_index, o, hd ** -0.5, 0, nH, nKV, hd,
+                                                     PAGE, T, ctx))
+    pairs = n_seqs * (ctx if decode else T * (T + 1) // 2)
+    att_work = n_seqs * ctx * nKV * 2 * hd * 2 if decode else 4.0 * pairs * hd * nH
+    seen = set()
+    for kind, m, _ in sh["layers"]:
+        if kind in seen:
+            continue
+        seen.add(kind)
+        if kind == "latent_attention":
+            H, rank, vdim = m["heads"], m["kv_rank"], m["vdim"]
+            qa = rnd(rows, H * rank)
+            gate = rnd(rows, H)
+            lat_pool = rnd(n_seqs * pages, PAGE * rank)
+            mixed = torch.empty((rows, H * rank), dtype=bf, device=dev)
+            t_new = _timed_graph(lambda: ops.attend_masked(
+                qa, gate, "head", lat_pool, None, None, table, q_start, ctx_len, seq_index, mixed,
+                m["scale"], 0.0, 0, 0, H, 1, rank, rank, PAGE, T, ctx))
+            new_work = n_seqs * ctx * rank * 2 if decode else 4.0 * pairs * rank * H
+            row("latent_attention", t_new, new_work, mat_rate, mat_bound, t_att, att_work,
+                mat_rate, mat_bound)
+            qfull = rnd(rows, H * m["dim"])
+            uk_t, uv = rnd(H, rank, m["dim"]), rnd(H, vdim, rank)
+            attn = torch.empty((rows, H * vdim), dtype=bf, device=dev)
+
+            def around():
+                ops.head_products(qfull, 0, m["dim"], uk_t, None, qa, 0, rank)
+                ops.head_products(mixed, 0, rank, uv, None, attn, 0, vdim)
+            t_hp = _timed_graph(around)
+            work = H * rank * (m["dim"] + vdim) * 2 if decode \
+                else 2.0 * rows * H * rank * (m["dim"] + vdim)
+            row("head_products", t_hp, work, mat_rate, mat_bound)
+            continue
+        H, d = m["heads"], m["dim"]
+        dv = m.get("vdim", d)
+        size = ops.recurrence_state_size(H, d, dv)
+        state = torch.zeros((n_seqs, size + W), dtype=torch.float32, device=dev)
+        qk = rnd(2, rows, H * d)
+        v = rnd(rows, H * dv)
+        z = torch.randn((rows, H * d), generator=g, device=dev)
+        zb = torch.zeros((H * d,), device=dev)
+        bonus = torch.rand((H * d,), generator=g, device=dev) if kind == "wkv" else None
+        ro = torch.empty((rows, H * dv), dtype=torch.float32, device=dev)
+        rule = "double_exp" if kind == "wkv" else "sigmoid_root"
+        t_new = _timed_graph(lambda: ops.decay_recurrence(
+            qk[0], qk[1], v, z, zb, bonus, state, state_slots, q_start, ro, H, d, dv, rule,
+            tau=float(m.get("tau", 1.0)), q_scale=d ** -0.5))
+        if decode:
+            row(kind + "_recurrence", t_new, 2.0 * n_seqs * H * d * dv * 4, read_bw, "read",
+                t_att, att_work, read_bw, "read")
+        else:
+            row(kind + "_recurrence", t_new, 5.0 * rows * H * d * dv, PEAK_FLOPS["fp32"],
+                "fp32_vector", t_att, att_work, mfma_rate, "mfma")
+        gate = rnd(rows, H * dv)
+        gain = torch.ones((dv if kind == "gla" else H * dv,), device=dev)
+        mixed = torch.empty((rows, H * dv), dtype=bf, device=dev)
+        t_norm = _timed_graph(lambda: ops.head_norm_gate(ro, gain, gate, mixed, H, 1e-6))
+        row(kind + "_head_norm_gate", t_norm, rows * H * dv * (4 + 2 + 2), read_bw, "read")
+        if kind == "wkv":
+            h = rnd(rows, W)
+            mu = torch.rand((5, W), generator=g, device=dev)
+            mixes = torch.empty((5, rows, W), dtype=bf, device=dev)
+            t_mix = _timed_graph(lambda: ops.token_shift_mix(h, mu, state, size, state_slots,
+                                                             seq_index, q_start, mixes))
+            row("token_shift_mix", t_mix, rows * W * 2 * (1 + 5), read_bw, "read")
+    # ---- feed-forwards: two matrices around a squared relu beside three of 2/3 the width
+    h = rnd(rows, W)
+    branch = torch.zeros((rows, W), dtype=torch.float32, device=dev)
+    dense = next((f for _, _, f in sh["layers"] if f["kind"] == "dense"), None)
+    moe = next((f for _, _, f in sh["layers"] if f["kind"] == "moe"), None)
+
+    def gated_twin(inter):
+        wgu = ops.pretile_weight(ops.interleave_gate_up(rnd(inter, W), rnd(inter, W)))
+        wd = ops.pretile_weight(rnd(W, inter))
+        act2 = torch.empty((rows, inter), dtype=bf, device=dev)
+
+        def run():
+            ops.gemm_swiglu(h, wgu, act2, w_tiled=True)
+            ops.gemm(act2, wd, branch, accumulate=True, w_tiled=True)
+        return _timed_graph(run)
+    if dense is not None:
+        ff = dense["ff"]
+        w_up, w_down = ops.pretile_weight(rnd(ff, W)), ops.pretile_weight(rnd(W, ff))
+        act = torch.empty((rows, ff), dtype=bf, device=dev)
+
+        def plain_ff():
+            ops.gemm(h, w_up, act, w_tiled=True)
+            ops.activation(act, act, "relu2")
+            ops.gemm(act, w_down, branch, accumulate=True, w_tiled=True)
+        t_new = _timed_graph(plain_ff)
+        inter = ff * 2 // 3 // 64 * 64
+        t_old = gated_twin(inter)
+        if decode:
+            row("feed_forward", t_new, 2 * ff * W * 2, read_bw, "read", t_old, 3 * inter * W * 2,
+                read_bw, "read")
+        else:
+            row("feed_forward", t_new, 2.0 * rows * 2 * ff * W, mfma_rate, "mfma", t_old,
+                2.0 * rows * 3 * inter * W, mfma_rate, "mfma")
+    if moe is not None:
+        E, top, ff = moe["router"]["experts"], moe["router"]["top"], moe["expert"]["ff"]
+        groups = (moe["router"]["groups"]["count"], moe["router"]["groups"]["keep"])
+        router = torch.randn((E, W), generator=g, device=dev) * 0.05
+        correction = torch.randn((E,), generator=g, device=dev) * 0.1
+        ids = torch.empty((rows, top), dtype=torch.int32, device=dev)
+        share = torch.empty((rows, top), dtype=torch.float32, device=dev)
+        up, down = rnd(E, ff, W), rnd(E, W, ff)
+        y = torch.empty((rows, top, ff), dtype=bf, device=dev)
+
+        def mixture():
+            ops.moe_route(h, router, None, ids, share, scoring="sigmoid", correction=correction,
+                          groups=groups)
+            ops.moe_experts(h, up, down, ids, share, y, branch, 0.0, 1.0, 0.0, add=True,
+                            act="relu2")
+        t_new = _timed_graph(mixture)
+        inter = top * ff * 2 // 3 // 64 * 64
+        t_old = gated_twin(inter)
+        if decode:
+            used = min(E, rows * top)        # at most this many experts' matrices are read
+            row("mixture", t_new, used * 2 * ff * W * 2, read_bw, "read", t_old,
+                3 * inter * W * 2, read_bw, "read")
+        else:
+            row("mixture", t_new, 2.0 * rows * 2 * top * ff * W, mfma_rate, "mfma", t_old,
+                2.0 * rows * 3 * inter * W, mfma_rate, "mfma")
+    return out
+
+
+def main_nupovik(args) -> int:
+    """Prefill and decode throughput of Nupovik shapes beside the dense Qwen3 decoder of equal
+    size, and the new kernels alone beside the like kernels of that decoder."""
+    import torch
+    import zinfer_amd.ops as ops
+    from zinfer_amd.config import entry_for
+    T, batch, prompt = args.prefill_tokens, args.batch, args.prompt_len
+    max_positions = max(T, prompt + args.steps + args.warmup + 64) + 64
+    read_bw = ops.measure_read_bandwidth("cuda:0")
+    mfma_rate = ops.measure_mfma_rate("cuda:0")
+    names = [args.nupovik_shape] if args.nupovik_shape else list(NUPOVIK_SHAPES)
+    shapes = {}
+    for name in names:
+        sh = NUPOVIK_SHAPES[name]
+        row = {"sizes": {"width": sh["width"], "vocab": sh["vocab"], "loop": sh["loop"],
+                         "layers": [[k, m, f] for k, m, f in sh["layers"]]}}
+        for label, raw in (("nupovik", nupovik_config(sh)), ("qwen3", nupovik_twin(sh, max_positions))):
+            cfg = entry_for(raw).config_type.from_dict(raw)
+            pool = batch * (prompt + args.steps + args.warmup + 64) + T + 256
+            llm = build_llm(raw, args.dtype, args.seed, pool, max(batch, 8),
+                            max_step_tokens=max(T, 2048), multi_step=args.multi_step)
+            t_pre = run_prefill(llm, cfg, T, args.seed + 1)
+            dt, mean_ctx = run_decode(llm, cfg, batch, prompt, args.steps, args.warmup, args.seed + 2)
+            row[label] = {"prefill_tokens_per_s": round(T / t_pre, 1), "prefill_ms": round(t_pre * 1e3, 3),
+                          "decode_tokens_per_s": round(batch * args.steps / dt, 1),
+                          "decode_ms_per_step": round(dt / args.steps * 1e3, 4),
+                          "decode_mean_context": round(mean_ctx, 1)}
+            drop(llm)
+        row["prefill_vs_qwen3"] = round(row["nupovik"]["prefill_tokens_per_s"]
+                                        / row["qwen3"]["prefill_tokens_per_s"], 3)
+        row["decode_vs_qwen3"] = round(row["nupovik"]["decode_tokens_per_s"]
+                                       / row["qwen3"]["decode_tokens_per_s"], 3)
+        if args.dtype == "bfloat16":
+            row["kernels_prefill"] = nupovik_kernels(sh, T, T, mfma_rate, read_bw)
+            row["kernels_decode"] = nupovik_kernels(sh, 1, prompt, mfma_rate, read_bw)
+        ops._workspaces.clear()
+        torch.cuda.empty_cache()
+        shapes[name] = row
+    first = shapes[names[0]]
+    print(json.dumps({
+        "metric": "nupovik_decode_tokens_per_s", "value": first["nupovik"]["decode_tokens_per_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["nupovik"]["decode_ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic", "config": {"model": f"Nupovik {names[0]} shape beside the dense Qwen3 "
+                                                 "decoder of equal size, random weights",
+                                        "batch": batch, "prompt_len": prompt, "prefill_tokens": T,
+                                        "parallelism": "single GPU"},
+        "measured_read_gbs": round(read_bw / 1e9, 1), "mfma_loop_tflops": round(mfma_rate / 1e12, 1),
+        "shapes": shapes}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel", "lodenex"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel", "lodenex", "nupovik"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="layer sizes (default: 8b for decode, 14b for continuous, 32b for "
                          "long-context)")
@@ -1046,6 +1328,8 @@ def main() -> int:
                     help="fezupel: only this shape (default: all of them)")
     ap.add_argument("--lodenex-shape", default=None, choices=sorted(LODENEX_SHAPES),
                     help="lodenex: only this shape (default: gqa, latent and mixed)")
+    ap.add_argument("--nupovik-shape", default=None, choices=sorted(NUPOVIK_SHAPES),
+                    help="nupovik: only this shape (default: all of them)")
     ap.add_argument("--no-run-graphs", action="store_true",
                     help="decode steps in a row replay one graph per step instead of one for the run")
     args = ap.parse_args()
@@ -1055,7 +1339,7 @@ def main() -> int:
         return 2
     return {"decode": main_decode, "continuous": main_continuous,
             "long-context": main_long_context, "fezupel": main_fezupel,
-            "lodenex": main_lodenex}[args.workload](args)
+            "lodenex": main_lodenex, "nupovik": main_nupovik}[args.workload](args)
 
 
 if __name__ == "__main__":
