@@ -138,7 +138,10 @@ def test_replay_modes(name, dtype, mode):
 @pytest.mark.parametrize("name", sorted(nt.CONFIGS))
 def test_cut_and_batch_leave_the_bits(name):
     """32-bit: a position's logits are the same bits whole, in portions, token by token and
-    beside other requests, whichever slot and pages the request got."""
+    beside other requests, whichever slot and pages the request got.  A portion of more than two
+    spans of the recurrence runs its spans side by side: there the sums have another order, and
+    the logits agree to rounding."""
+    from zinfer_amd import ops
     requests = _requests(name)
     vocab = nt.CONFIGS[name]["vocab"]
     rows = []
@@ -148,7 +151,11 @@ def test_cut_and_batch_leave_the_bits(name):
         rows.append(traces.collect(steps, _replay(eng, steps), vocab))
     for other in rows[1:]:
         for rid in rows[0]:
-            assert np.array_equal(rows[0][rid], other[rid]), rid
+            if len(requests[rid]) <= 2 * ops.RECURRENCE_SPAN:
+                assert np.array_equal(rows[0][rid], other[rid]), rid
+            else:
+                scale = float(np.abs(rows[0][rid]).max())
+                assert float(np.abs(rows[0][rid] - other[rid]).max()) < 2e-5 * scale, rid
 
 
 def test_a_slot_that_is_used_again_starts_from_zero():

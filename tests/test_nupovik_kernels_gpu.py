@@ -133,8 +133,10 @@ def _plain_recurrence(q, k, v, z, bias, bonus, H, d, dv, rule, tau, q_scale, sta
     return o.reshape(T, H * dv), S
 
 
-def _run_recurrence(parts, state, slots, bias, bonus, H, d, dv, rule, tau, q_scale, dt, columns=None):
-    """``parts``: (q, k, v, z) a sequence for this step."""
+def _run_recurrence(parts, state, slots, bias, bonus, H, d, dv, rule, tau, q_scale, dt, columns=None,
+                    span=0):
+    """``parts``: (q, k, v, z) a sequence for this step.  ``span`` 0: token by token from end to
+    end; None: the spans the product chooses; else spans of that many tokens."""
     lens = [p[0].shape[0] for p in parts]
     cat = [torch.cat([p[i] for p in parts]) for i in range(4)]
     T = sum(lens)
@@ -142,7 +144,7 @@ def _run_recurrence(parts, state, slots, bias, bonus, H, d, dv, rule, tau, q_sca
     ops.decay_recurrence(cat[0].to(dt).to(DEV), cat[1].to(dt).to(DEV), cat[2].to(dt).to(DEV),
                          cat[3].to(DEV), bias.to(DEV), None if bonus is None else bonus.to(DEV),
                          state, _i32(slots), _i32(_starts(lens)), out, H, d, dv, rule, tau=tau,
-                         q_scale=q_scale, columns=columns)
+                         q_scale=q_scale, columns=columns, max_q_len=max(lens), span=span)
     return out.cpu(), _starts(lens)
 
 
@@ -204,6 +206,56 @@ def test_decay_recurrence_against_plain(dt, case):
     assert torch.equal(again, state)
 
 
+SPANNED = [  # H, d, dv, rule, bonus, tau, span, lens of the first step, lens of the second
+    (2, 12, 12, "double_exp", True, 1.0, 16, [33, 1, 80, 16, 49], [40, 2, 1, 33, 64]),
+    (3, 20, 9, "sigmoid_root", False, 4.0, 16, [100, 32, 17], [1, 97, 48]),
+    (1, 64, 40, "sigmoid_root", False, 16.0, 32, [200, 65], [129, 3]),
+    (2, 136, 8, "double_exp", True, 1.0, 16, [48, 50], [35, 1]),
+    (4, 8, 16, "double_exp", True, 1.0, None, [300, 129, 5], [130, 1, 260]),
+    (1, 7, 3, "sigmoid_root", True, 2.5, 48, [150], [97]),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", SPANNED)
+def test_decay_recurrence_in_spans(dt, case):
+    """Portions of several spans beside portions of one span and single tokens, in one launch:
+    lengths that end at a span's edge, one token behind it and one before it.  Two steps: the
+    second starts from the states the first left and leaves its own."""
+    H, d, dv, rule, with_bonus, tau, span, first, second = case
+    q_scale = d ** -0.5
+    seqs = []
+    for i, n in enumerate(a + b for a, b in zip(first, second)):
+        q, k = _rand((n, H * d), 100 + i, 1.0, dt), _rand((n, H * d), 200 + i, 1.0, dt)
+        seqs.append((q, k, _rand((n, H * dv), 300 + i, 1.0, dt), _rand((n, H * d), 400 + i, 2.0)))
+    bias = _rand((H * d,), 5, 1.0) + (2.0 if rule == "sigmoid_root" else -2.0)
+    bonus = _rand((H * d,), 6, 0.5) if with_bonus else None
+    size = ops.recurrence_state_size(H, d, dv)
+    state = torch.zeros((len(seqs) + 1, size + 3), dtype=torch.float32, device=DEV)
+    slots = list(range(len(seqs), 0, -1))
+    heads = [tuple(t[:c] for t in s) for s, c in zip(seqs, first)]
+    tails = [tuple(t[c:] for t in s) for s, c in zip(seqs, first)]
+    o1, a1 = _run_recurrence(heads, state, slots, bias, bonus, H, d, dv, rule, tau, q_scale, dt,
+                             span=span)
+    limit = 2e-5 if dt == torch.float32 else 2.0 ** -7
+    for i, (s, c) in enumerate(zip(seqs, first)):
+        want, S = _plain_recurrence(*(t[:c] for t in s), bias, bonus, H, d, dv, rule, tau, q_scale)
+        assert rel_err(o1[a1[i]:a1[i + 1]], want) < limit, i
+        assert rel_err(ops.recurrence_state_matrix(state[slots[i]], H, d, dv), S) < 2e-5, i
+    order = list(reversed(range(len(seqs))))        # the second step lists the requests backwards
+    o2, a2 = _run_recurrence([tails[i] for i in order], state, [slots[i] for i in order], bias,
+                             bonus, H, d, dv, rule, tau, q_scale, dt, span=span)
+    for j, i in enumerate(order):
+        want, S = _plain_recurrence(*seqs[i], bias, bonus, H, d, dv, rule, tau, q_scale)
+        assert rel_err(o2[a2[j]:a2[j + 1]], want[first[i]:]) < limit, i
+        assert rel_err(ops.recurrence_state_matrix(state[slots[i]], H, d, dv), S) < 2e-5, i
+    assert float(state[0].abs().max()) == 0.0 and float(state[:, size:].abs().max()) == 0.0
+    # against the walk from end to end: rounding apart, the same
+    again = torch.zeros_like(state)
+    w1, _ = _run_recurrence(heads, again, slots, bias, bonus, H, d, dv, rule, tau, q_scale, dt)
+    assert rel_err(o1, w1) < 1e-5
+
+
 @pytest.mark.parametrize("rule", ["sigmoid_root", "double_exp"])
 def test_a_token_far_back_is_kept_or_lost_by_its_channel(rule):
     """Channel 0 does not decay, channel 1 decays fast.  A key on channel 0 at position 2 with
@@ -226,13 +278,15 @@ def test_a_token_far_back_is_kept_or_lost_by_its_channel(rule):
         z = torch.zeros((n, d))
         bonus = torch.zeros((d,)) if rule == "double_exp" else None
         want, _ = _plain_recurrence(q, k, v, z, bias, bonus, H, d, dv, rule, 1.0, 1.0)
-        for cut in (n, n - 1, 3, 2):              # whole; the last token alone; cut right behind the key
+        # whole; the last token alone; cut right behind the key; each token by token and in spans
+        for cut, span in ((n, 0), (n, None), (n, 16), (n - 1, None), (3, 0), (3, None), (2, 0)):
             state = torch.zeros((1, ops.recurrence_state_size(H, d, dv)), device=DEV)
             outs = []
             for a, b in ((0, cut), (cut, n)):
                 if a < b:
                     o, _ = _run_recurrence([(q[a:b], k[a:b], v[a:b], z[a:b])], state, [0], bias,
-                                           bonus, H, d, dv, rule, 1.0, 1.0, torch.float32)
+                                           bonus, H, d, dv, rule, 1.0, 1.0, torch.float32,
+                                           span=span)
                     outs.append(o)
             got = torch.cat(outs)
             assert rel_err(got, want) < 2e-5

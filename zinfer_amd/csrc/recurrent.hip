@@ -16,13 +16,18 @@
 //                        which then takes the portion's last row
 //  * decay_recurrence    the recurrence, token by token; a request's state is read at the start
 //                        of its portion and written at its end
+//  * decay_recurrence_spans   the same for long portions, cut into spans that run side by side:
+//                        every span's own sum from a zero state, then the states at the spans'
+//                        starts one after the other (S <- diag(product of the span's decays) S +
+//                        the span's sum), then every span's outputs from the state at its start
 //  * head_norm_gate      out = o / rms_head(o) * gain * silu(g)
 #include "zf_common.h"
 
 // ---------------------------------------------------------------- token shift
-// grid (token), any block: mixes [n_mix][T][W] in the rows' type.  The workgroup of a portion's
-// first token reads the state row and is the one that overwrites it (with the portion's last
-// row), element by element in the thread that read it: no other workgroup touches that row.
+// grid (token, block of columns), an element a thread: mixes [n_mix][T][W] in the rows' type.
+// The workgroups of a portion's first token read the state row and are the ones that overwrite
+// it (with the portion's last row), element by element in the thread that read it: no other
+// thread touches that element.
 template <typename T>
 __global__ void token_shift_mix_kernel(const T* __restrict__ h, const float* __restrict__ mu,
                                        float* __restrict__ state, long long slot_stride,
@@ -38,7 +43,8 @@ __global__ void token_shift_mix_kernel(const T* __restrict__ h, const float* __r
   const T* before = first ? nullptr : row - W;
   float* st = state + (size_t)state_slots[s] * slot_stride;
   const T* last = h + (size_t)(t1 - 1) * W;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i < W) {
     const float x = load_as_float<T>(row + i);
     const float p = first ? st[i] : load_as_float<T>(before + i);
     const float dx = p - x;
@@ -56,12 +62,13 @@ extern "C" int zf_token_shift_mix(const void* h, int dtype, const float* mu, flo
   if (T <= 0) return 0;
   if (W <= 0 || n_mix <= 0) return -2;
   const int block = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+  const dim3 grid(T, (W + block - 1) / block);
   if (dtype == ZF_F32)
-    hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(T), dim3(block), 0, stream,
+    hipLaunchKernelGGL(token_shift_mix_kernel<float>, grid, dim3(block), 0, stream,
                        (const float*)h, mu, state, slot_stride, state_slots, seq_index, q_start,
                        (float*)out, T, W, n_mix);
   else
-    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, dim3(T), dim3(block), 0, stream,
+    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, grid, dim3(block), 0, stream,
                        (const bf16_t*)h, mu, state, slot_stride, state_slots, seq_index, q_start,
                        (bf16_t*)out, T, W, n_mix);
   ZF_CHECK_LAUNCH();
@@ -79,7 +86,16 @@ __device__ __forceinline__ float decay_of(float z, int rule, float inv_tau) {
     const float sp = fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
     return expf(-sp * inv_tau);
   }
+  if (rule == 2) return z;                // the decays themselves
   return expf(-expf(z));
+}
+
+// z <- the decays of z, in place, an element a thread: spans of a portion then read them as they
+// are (rule 2) instead of each forming them again.
+__global__ void decays_in_place_kernel(float* __restrict__ z, const float* __restrict__ z_bias,
+                                       long long n, int width, int rule, float inv_tau) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) z[i] = decay_of(z[i] + z_bias[i % width], rule, inv_tau);
 }
 
 // grid (sequence, head, block of VB value columns); thread (vl, cg) = (tid / CS, tid % CS)
@@ -87,14 +103,22 @@ __device__ __forceinline__ float decay_of(float z, int rule, float inv_tau) {
 // channels a thread holds lie side by side (channels beyond d are padding that stays zero).
 // A token's partial outputs (one a thread) go to LDS and are added in ascending cg, so the sum
 // over channels has one order whatever VB is and however a prompt is cut.
-template <typename T, bool BEFORE>
+//
+// MODE 0: a sequence's whole portion in one workgroup.  With spans of ``span`` tokens
+// (blockIdx.x = sequence * max_spans + span number): MODE 1 runs a span from a zero state, writes
+// no output and leaves the span's sum in span_state and the product of its decays in span_decay
+// (the workgroups of value block 0 do); MODE 2 starts from span_state (by then the state at the
+// span's start) and writes the outputs.  A sequence of a single span is left alone by MODE 1 and
+// runs as in MODE 0 under MODE 2.
+template <typename T, bool BEFORE, int MODE>
 __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride,
     const T* __restrict__ v, long long v_stride, const float* __restrict__ z,
     const float* __restrict__ z_bias, const float* __restrict__ bonus,
     float* __restrict__ state, long long slot_stride, const int* __restrict__ state_slots,
     const int* __restrict__ q_start, float* __restrict__ out, int H, int d, int dv, int CS,
-    int VB, int TC, int rule, float inv_tau, float q_scale) {
+    int VB, int TC, int rule, float inv_tau, float q_scale, int span, int max_spans,
+    float* __restrict__ span_state, float* __restrict__ span_decay) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int DP = CS * REC_R;
   float* qs = lds;                        // [TC][DP]
@@ -103,18 +127,34 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
   float* us = ds + TC * DP;               // [DP]
   float* vs = us + DP;                    // [TC][VB]
   float* po = vs + TC * VB;               // [TC][VB][CS]
-  const int s = blockIdx.x, hd = blockIdx.y, v0 = blockIdx.z * VB;
-  const int t0 = q_start[s], t1 = q_start[s + 1];
+  float* pd = po + TC * VB * CS;          // [DP], MODE 1: the product of the span's decays
+  const int hd = blockIdx.y, v0 = blockIdx.z * VB;
+  int s = blockIdx.x, t0, t1;
+  bool alone = true;                      // the portion is this workgroup's from end to end
+  if (MODE == 0) {
+    t0 = q_start[s], t1 = q_start[s + 1];
+  } else {
+    s = blockIdx.x / max_spans;
+    const int a = q_start[s], b = q_start[s + 1];
+    alone = b - a <= span;
+    t0 = a + (blockIdx.x % max_spans) * span;
+    t1 = min(b, t0 + span);
+    if (MODE == 1 && alone) return;
+  }
   if (t0 >= t1) return;
   const int tid = threadIdx.x, nthreads = blockDim.x;
   const int vl = tid / CS, cg = tid % CS;
   const bool mine = vl < VB && v0 + vl < dv;
-  float* st = state + (size_t)state_slots[s] * slot_stride +
-              ((size_t)hd * dv + v0 + vl) * DP + cg * REC_R;
+  const size_t mine_at = ((size_t)hd * dv + v0 + vl) * DP + cg * REC_R;
+  float* st = state + (size_t)state_slots[s] * slot_stride + mine_at;
+  if (!alone) st = span_state + (size_t)blockIdx.x * ((size_t)H * dv * DP) + mine_at;
+  const bool decays_out = MODE == 1 && blockIdx.z == 0;
+  if (decays_out)
+    for (int c = tid; c < DP; c += nthreads) pd[c] = 1.f;
   float S[REC_R];
 #pragma unroll
   for (int j = 0; j < REC_R; ++j) S[j] = 0.f;
-  if (mine) {
+  if (mine && MODE != 1) {
     const float4 a = *(const float4*)st, b = *(const float4*)(st + 4);
     S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w;
     S[4] = b.x; S[5] = b.y; S[6] = b.z; S[7] = b.w;
@@ -129,9 +169,10 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
       float qv = 0.f, kv = 0.f, dc = 1.f;
       if (c < d) {
         const size_t row = (size_t)(tc + t);
-        qv = load_as_float<T>(q + row * q_stride + hd * d + c) * q_scale;
+        if (MODE != 1) qv = load_as_float<T>(q + row * q_stride + hd * d + c) * q_scale;
         kv = load_as_float<T>(k + row * k_stride + hd * d + c);
-        dc = decay_of(z[row * ((size_t)H * d) + hd * d + c] + z_bias[hd * d + c], rule, inv_tau);
+        const float zv = z[row * ((size_t)H * d) + hd * d + c];
+        dc = rule == 2 ? zv : decay_of(zv + z_bias[hd * d + c], rule, inv_tau);
       }
       qs[i] = qv; ks[i] = kv; ds[i] = dc;
     }
@@ -141,6 +182,27 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
                           : 0.f;
     }
     __syncthreads();
+    if (decays_out)
+      for (int c = tid; c < DP; c += nthreads) {
+        float p = pd[c];
+        for (int t = 0; t < n; ++t) p *= ds[t * DP + c];
+        pd[c] = p;
+      }
+    if (MODE == 1) {
+      if (vl < VB) {
+        for (int t = 0; t < n; ++t) {
+          const float vv = vs[t * VB + vl];
+          const float4* kp = (const float4*)(ks + t * DP + cg * REC_R);
+          const float4* dp = (const float4*)(ds + t * DP + cg * REC_R);
+          const float4 k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
+          const float k8[REC_R] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+          const float d8[REC_R] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+#pragma unroll
+          for (int j = 0; j < REC_R; ++j) S[j] = fmaf(d8[j], S[j], k8[j] * vv);
+        }
+      }
+      continue;
+    }
     if (vl < VB) {
       for (int t = 0; t < n; ++t) {
         const float vv = vs[t * VB + vl];
@@ -181,10 +243,42 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
       out[(size_t)(tc + t) * ((size_t)H * dv) + hd * dv + v0 + x] = sum;
     }
   }
-  if (mine) {
+  if (mine && (MODE == 1 || alone)) {
     *(float4*)st = float4{S[0], S[1], S[2], S[3]};
     *(float4*)(st + 4) = float4{S[4], S[5], S[6], S[7]};
   }
+  if (decays_out)                         // each thread wrote the entries it reads here
+    for (int c = tid; c < DP; c += nthreads)
+      span_decay[((size_t)blockIdx.x * H + hd) * DP + c] = pd[c];
+}
+
+// The states at the spans' starts, one after the other: a thread keeps 4 neighbouring entries of
+// a sequence's state (same head, same value column), walks the sequence's spans, leaves in
+// span_state[n] the state before span n where the span's own sum was, and writes the state behind
+// the last span to the request's slot.  grid (ceil(size / 4 / 256), sequence).
+__global__ __launch_bounds__(256) void span_states_kernel(
+    float* __restrict__ state, long long slot_stride, const int* __restrict__ state_slots,
+    const int* __restrict__ q_start, float* __restrict__ span_state,
+    const float* __restrict__ span_decay, int H, int dv, int DP, int span, int max_spans) {
+  const int s = blockIdx.y;
+  const int len = q_start[s + 1] - q_start[s];
+  if (len <= span) return;
+  const int n_spans = (len + span - 1) / span;
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (e >= (long long)H * dv * DP) return;
+  const int hd = (int)(e / ((long long)dv * DP)), c = (int)(e % DP);
+  float* st = state + (size_t)state_slots[s] * slot_stride + e;
+  float4 S = *(const float4*)st;
+  for (int n = 0; n < n_spans; ++n) {
+    const size_t w = (size_t)s * max_spans + n;
+    float4* at = (float4*)(span_state + w * ((size_t)H * dv * DP) + e);
+    const float4 own = *at;
+    const float4 dc = *(const float4*)(span_decay + (w * H + hd) * DP + c);
+    *at = S;
+    S = float4{fmaf(dc.x, S.x, own.x), fmaf(dc.y, S.y, own.y), fmaf(dc.z, S.z, own.z),
+               fmaf(dc.w, S.w, own.w)};
+  }
+  *(float4*)st = S;
 }
 
 // q, k [T, >= H d], v [T, >= H dv] with contiguous rows (strides in elements), z [T, H d] and
@@ -204,20 +298,60 @@ extern "C" int zf_decay_recurrence(const void* q, long long q_stride, const void
     return -2;
   const int DP = CS * REC_R;
   const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
-  const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + DP + (size_t)TC * VB +
+  const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + 2 * DP + (size_t)TC * VB +
                                        (size_t)TC * VB * CS);
   const int threads = (CS * VB + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
   const dim3 grid(n_seqs, H, (dv + VB - 1) / VB), block(threads);
-#define REC_LAUNCH(TT, BEF)                                                                      \
-  hipLaunchKernelGGL((decay_recurrence_kernel<TT, BEF>), grid, block, smem, stream,              \
+#define REC_LAUNCH(TT, BEF, MODE, GRID, RULE, SPAN, MAXS, SST, SDC)                              \
+  hipLaunchKernelGGL((decay_recurrence_kernel<TT, BEF, MODE>), GRID, block, smem, stream,        \
                      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z,  \
                      z_bias, bonus, state, slot_stride, state_slots, q_start, out, H, d, dv, CS, \
-                     VB, TC, rule, inv_tau, q_scale)
-  if (dtype == ZF_F32) {
-    if (bonus != nullptr) REC_LAUNCH(float, true); else REC_LAUNCH(float, false);
-  } else {
-    if (bonus != nullptr) REC_LAUNCH(bf16_t, true); else REC_LAUNCH(bf16_t, false);
+                     VB, TC, RULE, inv_tau, q_scale, SPAN, MAXS, SST, SDC)
+#define REC_LAUNCH_ANY(MODE, GRID, RULE, SPAN, MAXS, SST, SDC)                                   \
+  if (dtype == ZF_F32) {                                                                         \
+    if (bonus != nullptr) REC_LAUNCH(float, true, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);       \
+    else REC_LAUNCH(float, false, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);                       \
+  } else {                                                                                       \
+    if (bonus != nullptr) REC_LAUNCH(bf16_t, true, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);      \
+    else REC_LAUNCH(bf16_t, false, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);                      \
   }
+  REC_LAUNCH_ANY(0, grid, rule, 0, 1, nullptr, nullptr)
+  ZF_CHECK_LAUNCH();
+}
+
+// The same for portions cut into spans of ``span`` tokens (a multiple of 16), at most max_spans a
+// sequence.  z [T, H d] is overwritten with the decays.  span_state float32 [n_seqs * max_spans,
+// H dv padded d] and span_decay float32 [n_seqs * max_spans, H, padded d] are scratch.
+extern "C" int zf_decay_recurrence_spans(const void* q, long long q_stride, const void* k,
+                                         long long k_stride, const void* v, long long v_stride,
+                                         int dtype, float* z, const float* z_bias,
+                                         const float* bonus, float* state, long long slot_stride,
+                                         const int* state_slots, const int* q_start, float* out,
+                                         int n_tokens, int n_seqs, int H, int d, int dv, int VB,
+                                         int rule, float inv_tau, float q_scale, int span,
+                                         int max_spans, float* span_state, float* span_decay,
+                                         hipStream_t stream) {
+  if (n_seqs <= 0 || n_tokens <= 0) return 0;
+  const int CS = (d + REC_R - 1) / REC_R;
+  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 || CS * VB > REC_MAX_THREADS ||
+      rule < 0 || rule > 1 || slot_stride < (long long)H * dv * CS * REC_R || span < REC_TC || span % REC_TC != 0 || max_spans < 1 ||
+      span_state == nullptr || span_decay == nullptr)
+    return -2;
+  const int DP = CS * REC_R;
+  const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
+  const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + 2 * DP + (size_t)TC * VB +
+                                       (size_t)TC * VB * CS);
+  const int threads = (CS * VB + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
+  const dim3 grid(n_seqs * max_spans, H, (dv + VB - 1) / VB), block(threads);
+  const long long n = (long long)n_tokens * H * d;
+  hipLaunchKernelGGL(decays_in_place_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     stream, z, z_bias, n, H * d, rule, inv_tau);
+  REC_LAUNCH_ANY(1, grid, 2, span, max_spans, span_state, span_decay)
+  const long long quads = (long long)H * dv * DP / 4;
+  hipLaunchKernelGGL(span_states_kernel, dim3((unsigned)((quads + 255) / 256), n_seqs), dim3(256),
+                     0, stream, state, slot_stride, state_slots, q_start, span_state, span_decay,
+                     H, dv, DP, span, max_spans);
+  REC_LAUNCH_ANY(2, grid, 2, span, max_spans, span_state, span_decay)
   ZF_CHECK_LAUNCH();
 }
 

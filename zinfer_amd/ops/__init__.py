@@ -2313,6 +2313,8 @@ RECURRENCE_CHANNELS = 8          # REC_R in recurrent.hip: key channels a thread
 RECURRENCE_MAX_KEY_DIM = 256
 RECURRENCE_MAX_THREADS = 256
 RECURRENCE_WORKGROUPS = 512      # value columns are dealt over workgroups until about this many run
+RECURRENCE_SPAN = 64             # tokens of a span; a multiple of the 16 tokens the kernel stages
+RECURRENCE_MAX_SPANS = 64        # longer portions have longer spans instead of more
 DECAY_RULES = {"sigmoid_root": 0, "double_exp": 1}
 
 
@@ -2378,7 +2380,8 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
                      z_bias: torch.Tensor, bonus: Optional[torch.Tensor], state: torch.Tensor,
                      state_slots: torch.Tensor, q_start: torch.Tensor, out: torch.Tensor,
                      n_heads: int, key_dim: int, value_dim: int, rule: str, tau: float = 1.0,
-                     q_scale: float = 1.0, columns: Optional[int] = None) -> None:
+                     q_scale: float = 1.0, columns: Optional[int] = None,
+                     max_q_len: Optional[int] = None, span: Optional[int] = None) -> None:
     """The recurrence S_t = diag(a_t) S_(t-1) + k_t v_t^T a head, token by token in 32-bit, over
     the rows of a step: ``q``, ``k`` [T, H * d] and ``v`` [T, H * dv] (contiguous rows, any row
     stride), ``z`` float32 [T, H * d] with a_t = sigmoid(z_t + z_bias)^(1 / tau) (``rule``
@@ -2388,7 +2391,15 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
     Sequence s owns the rows q_start[s] .. q_start[s + 1] - 1; its state (row state_slots[s] of
     ``state``, float32 [slots, >= ``recurrence_state_size``]) is read before its first row and
     written behind its last.  A row's result depends on the state and the rows of its own
-    sequence alone, and not on how the sequence was cut into steps."""
+    sequence alone, and not on how the sequence was cut into steps, beyond rounding.
+
+    ``max_q_len``: the most rows a sequence has in this step, where the caller knows it.  Above
+    two spans (``span`` tokens, by default ``RECURRENCE_SPAN`` or what keeps a sequence within
+    ``RECURRENCE_MAX_SPANS``) the portions are cut into spans that run side by side: each span's
+    own sum from a zero state, the states at the spans' starts one after the other
+    (S <- diag(product of the span's decays) S + the span's sum), then each span's outputs from
+    the state at its start.  The same numbers up to 32-bit rounding; ``z`` is then overwritten
+    with the decays.  ``span`` 0, or no ``max_q_len``: token by token from end to end."""
     _need_gpu(z, z_bias, bonus, state, state_slots, q_start, out)
     for t in (q, k, v):
         if not t.is_cuda:
@@ -2413,8 +2424,32 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
                                 f"{tuple(out.shape)} {out.dtype}, state {tuple(state.shape)} for "
                                 f"{H} heads of {d} x {dv} (key size up to "
                                 f"{RECURRENCE_MAX_KEY_DIM}), rule {rule!r}")
-    vb = int(columns) if columns is not None else _recurrence_columns(n_seqs, H, d, dv)
     lib = build.load("recurrent")
+    longest = int(max_q_len) if max_q_len is not None else 0
+    if span is None:
+        span = RECURRENCE_SPAN
+        if longest > span * RECURRENCE_MAX_SPANS:
+            span = ((longest + RECURRENCE_MAX_SPANS - 1) // RECURRENCE_MAX_SPANS + 15) // 16 * 16
+    if span and (span % 16 or span < 16):
+        raise KernelUnavailable(f"decay_recurrence: a span of {span} tokens is no multiple of 16")
+    if span and longest > 2 * span and z.is_contiguous():
+        max_spans = (longest + span - 1) // span
+        works = n_seqs * max_spans
+        vb = int(columns) if columns is not None else _recurrence_columns(works, H, d, dv)
+        span_state = _workspace("recurrence_span_state", works * need, torch.float32, q.device)
+        span_decay = _workspace("recurrence_span_decay", works * (need // dv), torch.float32,
+                                q.device)
+        code = lib.zf_decay_recurrence_spans(
+            _ptr(q), ctypes.c_longlong(_columns(q, "decay_recurrence: q")), _ptr(k),
+            ctypes.c_longlong(_columns(k, "decay_recurrence: k")), _ptr(v),
+            ctypes.c_longlong(_columns(v, "decay_recurrence: v")), _dt(q), _ptr(z), _ptr(z_bias),
+            _ptr(bonus), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(state_slots),
+            _ptr(q_start), _ptr(out), T, n_seqs, H, d, dv, vb, DECAY_RULES[rule],
+            ctypes.c_float(1.0 / tau), ctypes.c_float(q_scale), int(span), max_spans,
+            _ptr(span_state), _ptr(span_decay), _stream())
+        _check(code, "decay_recurrence_spans")
+        return
+    vb = int(columns) if columns is not None else _recurrence_columns(n_seqs, H, d, dv)
     code = lib.zf_decay_recurrence(
         _ptr(q), ctypes.c_longlong(_columns(q, "decay_recurrence: q")), _ptr(k),
         ctypes.c_longlong(_columns(k, "decay_recurrence: k")), _ptr(v),

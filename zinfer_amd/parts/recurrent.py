@@ -33,8 +33,9 @@ class GatedLinearAttention(Mixer):
     """The mixer of ``GatedLinearAttentionSpec``: q, k, v and the output gate come from one
     product over the stacked matrices (each output keeps its own dot product); the decay's
     numbers z = W_a2 (W_a1 h) leave their product as 32-bit numbers, and the recurrence kernel
-    turns them into decays, walks the step's tokens and keeps every request's matrices in its
-    state slot (32-bit); one more kernel norms each head, applies the gain and the gate."""
+    turns them into decays, walks the step's tokens (long portions in spans side by side) and
+    keeps every request's matrices in its state slot (32-bit); one more kernel norms each head,
+    applies the gain and the gate."""
     graph_safe = True
     kernel_modules = ("gemm", "recurrent")
 
@@ -94,7 +95,7 @@ class GatedLinearAttention(Mixer):
         ops.decay_recurrence(proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], z,
                              self.decay_bias, None, cache.state, step.state_slots, step.q_start,
                              o, s.n_heads, s.head_dim, s.value_dim, "sigmoid_root",
-                             tau=float(s.tau), q_scale=self.q_scale)
+                             tau=float(s.tau), q_scale=self.q_scale, max_q_len=step.max_q_len)
         mixed = step.scratch("rec_mixed", (T, V), act)
         ops.head_norm_gate(o, self.gain, proj[:, 2 * QK + V:], mixed, s.n_heads,
                            float(s.norm_eps))
@@ -171,7 +172,7 @@ class TokenShiftRecurrence(Mixer):
         o = step.scratch("rec_out", (T, self.width), torch.float32)
         ops.decay_recurrence(rkvg[0], rkvg[1], rkvg[2], z, self.decay_bias, self.bonus,
                              cache.state, step.state_slots, step.q_start, o, s.n_heads,
-                             s.head_dim, s.head_dim, "double_exp")
+                             s.head_dim, s.head_dim, "double_exp", max_q_len=step.max_q_len)
         mixed = step.scratch("rec_mixed", (T, self.width), act)
         ops.head_norm_gate(o, self.gain, rkvg[3], mixed, s.n_heads, float(s.norm_eps))
         self.o.forward(mixed, residual, accumulate=True, step=step)
