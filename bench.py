@@ -1154,7 +1154,7 @@ def nupovik_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float
         rule = "double_exp" if kind == "wkv" else "sigmoid_root"
         t_new = _timed_graph(lambda: ops.decay_recurrence(
             qk[0], qk[1], v, z, zb, bonus, state, state_slots, q_start, ro, H, d, dv, rule,
-            tau=float(m.get("tau", 1.0)), q_scale=d ** -0.5))
+            tau=float(m.get("tau", 1.0)), q_scale=d ** -0.5, max_q_len=T))
         if decode:
             row(kind + "_recurrence", t_new, 2.0 * n_seqs * H * d * dv * 4, read_bw, "read",
                 t_att, att_work, read_bw, "read")

@@ -78,6 +78,7 @@ extern "C" int zf_token_shift_mix(const void* h, int dtype, const float* mu, flo
 #define REC_R 8            // key channels of a value column a thread keeps in registers
 #define REC_TC 16          // tokens staged at a time (half of that for more than 128 channels)
 #define REC_MAX_THREADS 256
+#define REC_MAX_LDS 65536
 
 __device__ __forceinline__ float decay_of(float z, int rule, float inv_tau) {
   if (rule == 0) {
@@ -99,10 +100,13 @@ __global__ void decays_in_place_kernel(float* __restrict__ z, const float* __res
 }
 
 // grid (sequence, head, block of VB value columns); thread (vl, cg) = (tid / CS, tid % CS)
-// holds S[8 cg .. 8 cg + 8, v0 + vl].  A request's state is laid out [head][dv][CS * 8]: the
-// channels a thread holds lie side by side (channels beyond d are padding that stays zero).
-// A token's partial outputs (one a thread) go to LDS and are added in ascending cg, so the sum
-// over channels has one order whatever VB is and however a prompt is cut.
+// holds S[8 cg .. 8 cg + 8, v0 + RV vl .. + RV]: RV value columns (4, 2 or 1: what divides VB),
+// so that a token's q, k and decays, read from LDS once, serve RV columns.  A request's state is
+// laid out [head][dv][CS * 8]: the channels a thread holds lie side by side (channels beyond d
+// are padding that stays zero).  A token's partial outputs (one a thread and column) go to LDS
+// (rows of CS, padded to an odd length so that the sums' reads spread over the banks) and are
+// added in ascending cg, so the sum over channels has one order whatever VB is and however a
+// prompt is cut.
 //
 // MODE 0: a sequence's whole portion in one workgroup.  With spans of ``span`` tokens
 // (blockIdx.x = sequence * max_spans + span number): MODE 1 runs a span from a zero state, writes
@@ -110,7 +114,7 @@ __global__ void decays_in_place_kernel(float* __restrict__ z, const float* __res
 // (the workgroups of value block 0 do); MODE 2 starts from span_state (by then the state at the
 // span's start) and writes the outputs.  A sequence of a single span is left alone by MODE 1 and
 // runs as in MODE 0 under MODE 2.
-template <typename T, bool BEFORE, int MODE>
+template <typename T, bool BEFORE, int MODE, int RV>
 __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride,
     const T* __restrict__ v, long long v_stride, const float* __restrict__ z,
@@ -121,13 +125,14 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
     float* __restrict__ span_state, float* __restrict__ span_decay) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int DP = CS * REC_R;
+  const int CSP = CS | 1;
   float* qs = lds;                        // [TC][DP]
   float* ks = qs + TC * DP;               // [TC][DP]
   float* ds = ks + TC * DP;               // [TC][DP]
   float* us = ds + TC * DP;               // [DP]
-  float* vs = us + DP;                    // [TC][VB]
-  float* po = vs + TC * VB;               // [TC][VB][CS]
-  float* pd = po + TC * VB * CS;          // [DP], MODE 1: the product of the span's decays
+  float* pd = us + DP;                    // [DP], MODE 1: the product of the span's decays
+  float* vs = pd + DP;                    // [TC][VB]
+  float* po = vs + TC * VB;               // [TC][VB][CSP]
   const int hd = blockIdx.y, v0 = blockIdx.z * VB;
   int s = blockIdx.x, t0, t1;
   bool alone = true;                      // the portion is this workgroup's from end to end
@@ -144,20 +149,25 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
   if (t0 >= t1) return;
   const int tid = threadIdx.x, nthreads = blockDim.x;
   const int vl = tid / CS, cg = tid % CS;
-  const bool mine = vl < VB && v0 + vl < dv;
-  const size_t mine_at = ((size_t)hd * dv + v0 + vl) * DP + cg * REC_R;
+  const int col = vl * RV;                // the thread's first column within the block
+  const bool active = col < VB;
+  const size_t mine_at = ((size_t)hd * dv + v0 + col) * DP + cg * REC_R;
   float* st = state + (size_t)state_slots[s] * slot_stride + mine_at;
   if (!alone) st = span_state + (size_t)blockIdx.x * ((size_t)H * dv * DP) + mine_at;
   const bool decays_out = MODE == 1 && blockIdx.z == 0;
   if (decays_out)
     for (int c = tid; c < DP; c += nthreads) pd[c] = 1.f;
-  float S[REC_R];
+  float S[RV][REC_R];
 #pragma unroll
-  for (int j = 0; j < REC_R; ++j) S[j] = 0.f;
-  if (mine && MODE != 1) {
-    const float4 a = *(const float4*)st, b = *(const float4*)(st + 4);
-    S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w;
-    S[4] = b.x; S[5] = b.y; S[6] = b.z; S[7] = b.w;
+  for (int r = 0; r < RV; ++r) {
+#pragma unroll
+    for (int j = 0; j < REC_R; ++j) S[r][j] = 0.f;
+    if (MODE != 1 && active && v0 + col + r < dv) {
+      const float4 a = *(const float4*)(st + (size_t)r * DP);
+      const float4 b = *(const float4*)(st + (size_t)r * DP + 4);
+      S[r][0] = a.x; S[r][1] = a.y; S[r][2] = a.z; S[r][3] = a.w;
+      S[r][4] = b.x; S[r][5] = b.y; S[r][6] = b.z; S[r][7] = b.w;
+    }
   }
   for (int c = tid; c < DP; c += nthreads)
     us[c] = (BEFORE && c < d) ? bonus[hd * d + c] : 0.f;
@@ -188,64 +198,71 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
         for (int t = 0; t < n; ++t) p *= ds[t * DP + c];
         pd[c] = p;
       }
-    if (MODE == 1) {
-      if (vl < VB) {
-        for (int t = 0; t < n; ++t) {
-          const float vv = vs[t * VB + vl];
-          const float4* kp = (const float4*)(ks + t * DP + cg * REC_R);
-          const float4* dp = (const float4*)(ds + t * DP + cg * REC_R);
-          const float4 k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
-          const float k8[REC_R] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-          const float d8[REC_R] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
-#pragma unroll
-          for (int j = 0; j < REC_R; ++j) S[j] = fmaf(d8[j], S[j], k8[j] * vv);
-        }
-      }
-      continue;
-    }
-    if (vl < VB) {
+    if (active) {
       for (int t = 0; t < n; ++t) {
-        const float vv = vs[t * VB + vl];
-        const float4* qp = (const float4*)(qs + t * DP + cg * REC_R);
+        float vv[RV];
+#pragma unroll
+        for (int r = 0; r < RV; ++r) vv[r] = vs[t * VB + col + r];
         const float4* kp = (const float4*)(ks + t * DP + cg * REC_R);
         const float4* dp = (const float4*)(ds + t * DP + cg * REC_R);
-        const float4 q0 = qp[0], q1 = qp[1], k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
-        const float q8[REC_R] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const float4 k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
         const float k8[REC_R] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
         const float d8[REC_R] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
-        float acc = 0.f;
+        if (MODE == 1) {
+#pragma unroll
+          for (int r = 0; r < RV; ++r)
+#pragma unroll
+            for (int j = 0; j < REC_R; ++j) S[r][j] = fmaf(d8[j], S[r][j], k8[j] * vv[r]);
+          continue;
+        }
+        const float4* qp = (const float4*)(qs + t * DP + cg * REC_R);
+        const float4 q0 = qp[0], q1 = qp[1];
+        const float q8[REC_R] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        float u8[REC_R];
         if (BEFORE) {
           const float4* up = (const float4*)(us + cg * REC_R);
           const float4 u0 = up[0], u1 = up[1];
-          const float u8[REC_R] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
-#pragma unroll
-          for (int j = 0; j < REC_R; ++j) {
-            const float kv = k8[j] * vv;
-            acc = fmaf(q8[j], fmaf(u8[j], kv, S[j]), acc);
-            S[j] = fmaf(d8[j], S[j], kv);
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < REC_R; ++j) {
-            S[j] = fmaf(d8[j], S[j], k8[j] * vv);
-            acc = fmaf(q8[j], S[j], acc);
-          }
+          u8[0] = u0.x; u8[1] = u0.y; u8[2] = u0.z; u8[3] = u0.w;
+          u8[4] = u1.x; u8[5] = u1.y; u8[6] = u1.z; u8[7] = u1.w;
         }
-        po[(t * VB + vl) * CS + cg] = acc;
+#pragma unroll
+        for (int r = 0; r < RV; ++r) {
+          float acc = 0.f;
+          if (BEFORE) {
+#pragma unroll
+            for (int j = 0; j < REC_R; ++j) {
+              const float kv = k8[j] * vv[r];
+              acc = fmaf(q8[j], fmaf(u8[j], kv, S[r][j]), acc);
+              S[r][j] = fmaf(d8[j], S[r][j], kv);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < REC_R; ++j) {
+              S[r][j] = fmaf(d8[j], S[r][j], k8[j] * vv[r]);
+              acc = fmaf(q8[j], S[r][j], acc);
+            }
+          }
+          po[(t * VB + col + r) * CSP + cg] = acc;
+        }
       }
     }
+    if (MODE == 1) continue;
     __syncthreads();
     for (int i = tid; i < n * VB; i += nthreads) {
       const int t = i / VB, x = i % VB;
       if (v0 + x >= dv) continue;
       float sum = 0.f;
-      for (int c = 0; c < CS; ++c) sum += po[i * CS + c];
+      for (int c = 0; c < CS; ++c) sum += po[i * CSP + c];
       out[(size_t)(tc + t) * ((size_t)H * dv) + hd * dv + v0 + x] = sum;
     }
   }
-  if (mine && (MODE == 1 || alone)) {
-    *(float4*)st = float4{S[0], S[1], S[2], S[3]};
-    *(float4*)(st + 4) = float4{S[4], S[5], S[6], S[7]};
+  if (MODE == 1 || alone) {
+#pragma unroll
+    for (int r = 0; r < RV; ++r)
+      if (active && v0 + col + r < dv) {
+        *(float4*)(st + (size_t)r * DP) = float4{S[r][0], S[r][1], S[r][2], S[r][3]};
+        *(float4*)(st + (size_t)r * DP + 4) = float4{S[r][4], S[r][5], S[r][6], S[r][7]};
+      }
   }
   if (decays_out)                         // each thread wrote the entries it reads here
     for (int c = tid; c < DP; c += nthreads)
@@ -282,8 +299,8 @@ __global__ __launch_bounds__(256) void span_states_kernel(
 }
 
 // q, k [T, >= H d], v [T, >= H dv] with contiguous rows (strides in elements), z [T, H d] and
-// out [T, H dv] float32, dense.  CS = ceil(d / 8) <= 32; VB value columns a workgroup,
-// CS * VB <= 256.
+// out [T, H dv] float32, dense.  CS = ceil(d / 8) <= 32; VB <= 256 value columns a workgroup,
+// RV of them a thread, CS * VB / RV <= 256.
 extern "C" int zf_decay_recurrence(const void* q, long long q_stride, const void* k,
                                    long long k_stride, const void* v, long long v_stride,
                                    int dtype, const float* z, const float* z_bias,
@@ -293,27 +310,34 @@ extern "C" int zf_decay_recurrence(const void* q, long long q_stride, const void
                                    float inv_tau, float q_scale, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   const int CS = (d + REC_R - 1) / REC_R;
-  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 || CS * VB > REC_MAX_THREADS ||
+  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 ||
+      CS * (VB / (VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1))) > REC_MAX_THREADS || VB > 256 ||
       rule < 0 || rule > 1 || slot_stride < (long long)H * dv * CS * REC_R)
     return -2;
   const int DP = CS * REC_R;
   const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
+  const int RV = VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1);
   const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + 2 * DP + (size_t)TC * VB +
-                                       (size_t)TC * VB * CS);
-  const int threads = (CS * VB + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
+                                       (size_t)TC * VB * (CS | 1));
+  if (smem > REC_MAX_LDS) return -2;
+  const int threads = (CS * (VB / RV) + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
   const dim3 grid(n_seqs, H, (dv + VB - 1) / VB), block(threads);
-#define REC_LAUNCH(TT, BEF, MODE, GRID, RULE, SPAN, MAXS, SST, SDC)                              \
-  hipLaunchKernelGGL((decay_recurrence_kernel<TT, BEF, MODE>), GRID, block, smem, stream,        \
+#define REC_LAUNCH_RV(TT, BEF, MODE, RVV, GRID, RULE, SPAN, MAXS, SST, SDC)                      \
+  hipLaunchKernelGGL((decay_recurrence_kernel<TT, BEF, MODE, RVV>), GRID, block, smem, stream,   \
                      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z,  \
                      z_bias, bonus, state, slot_stride, state_slots, q_start, out, H, d, dv, CS, \
                      VB, TC, RULE, inv_tau, q_scale, SPAN, MAXS, SST, SDC)
+#define REC_LAUNCH(TT, BEF, MODE, GRID, RULE, SPAN, MAXS, SST, SDC)                              \
+  if (RV == 4) REC_LAUNCH_RV(TT, BEF, MODE, 4, GRID, RULE, SPAN, MAXS, SST, SDC);                \
+  else if (RV == 2) REC_LAUNCH_RV(TT, BEF, MODE, 2, GRID, RULE, SPAN, MAXS, SST, SDC);           \
+  else REC_LAUNCH_RV(TT, BEF, MODE, 1, GRID, RULE, SPAN, MAXS, SST, SDC)
 #define REC_LAUNCH_ANY(MODE, GRID, RULE, SPAN, MAXS, SST, SDC)                                   \
   if (dtype == ZF_F32) {                                                                         \
-    if (bonus != nullptr) REC_LAUNCH(float, true, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);       \
-    else REC_LAUNCH(float, false, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);                       \
+    if (bonus != nullptr) { REC_LAUNCH(float, true, MODE, GRID, RULE, SPAN, MAXS, SST, SDC); }   \
+    else { REC_LAUNCH(float, false, MODE, GRID, RULE, SPAN, MAXS, SST, SDC); }                   \
   } else {                                                                                       \
-    if (bonus != nullptr) REC_LAUNCH(bf16_t, true, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);      \
-    else REC_LAUNCH(bf16_t, false, MODE, GRID, RULE, SPAN, MAXS, SST, SDC);                      \
+    if (bonus != nullptr) { REC_LAUNCH(bf16_t, true, MODE, GRID, RULE, SPAN, MAXS, SST, SDC); }  \
+    else { REC_LAUNCH(bf16_t, false, MODE, GRID, RULE, SPAN, MAXS, SST, SDC); }                  \
   }
   REC_LAUNCH_ANY(0, grid, rule, 0, 1, nullptr, nullptr)
   ZF_CHECK_LAUNCH();
@@ -333,15 +357,18 @@ extern "C" int zf_decay_recurrence_spans(const void* q, long long q_stride, cons
                                          hipStream_t stream) {
   if (n_seqs <= 0 || n_tokens <= 0) return 0;
   const int CS = (d + REC_R - 1) / REC_R;
-  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 || CS * VB > REC_MAX_THREADS ||
+  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 ||
+      CS * (VB / (VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1))) > REC_MAX_THREADS || VB > 256 ||
       rule < 0 || rule > 1 || slot_stride < (long long)H * dv * CS * REC_R || span < REC_TC || span % REC_TC != 0 || max_spans < 1 ||
       span_state == nullptr || span_decay == nullptr)
     return -2;
   const int DP = CS * REC_R;
   const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
+  const int RV = VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1);
   const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + 2 * DP + (size_t)TC * VB +
-                                       (size_t)TC * VB * CS);
-  const int threads = (CS * VB + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
+                                       (size_t)TC * VB * (CS | 1));
+  if (smem > REC_MAX_LDS) return -2;
+  const int threads = (CS * (VB / RV) + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
   const dim3 grid(n_seqs * max_spans, H, (dv + VB - 1) / VB), block(threads);
   const long long n = (long long)n_tokens * H * d;
   hipLaunchKernelGGL(decays_in_place_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,

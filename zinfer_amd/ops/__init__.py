@@ -2312,6 +2312,7 @@ def masked_attention_mfma(q, gate, gate_mode, k_pool, v_pool, sink, block_table,
 RECURRENCE_CHANNELS = 8          # REC_R in recurrent.hip: key channels a thread holds
 RECURRENCE_MAX_KEY_DIM = 256
 RECURRENCE_MAX_THREADS = 256
+RECURRENCE_MAX_LDS = 65536
 RECURRENCE_WORKGROUPS = 512      # value columns are dealt over workgroups until about this many run
 RECURRENCE_SPAN = 64             # tokens of a span; a multiple of the 16 tokens the kernel stages
 RECURRENCE_MAX_SPANS = 64        # longer portions have longer spans instead of more
@@ -2364,14 +2365,31 @@ def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, stat
            "token_shift_mix")
 
 
-def _recurrence_columns(n_seqs: int, n_heads: int, key_dim: int, value_dim: int) -> int:
-    """Value columns a workgroup of ``decay_recurrence`` takes: as many as its threads hold,
-    fewer where that leaves the chip idle.  The results do not depend on it."""
+def _recurrence_lds(key_dim: int, columns: int) -> int:
+    """Bytes of LDS a workgroup of ``decay_recurrence`` with ``columns`` value columns takes."""
     groups = (key_dim + RECURRENCE_CHANNELS - 1) // RECURRENCE_CHANNELS
-    most = max(1, min(value_dim, RECURRENCE_MAX_THREADS // groups))
+    padded = groups * RECURRENCE_CHANNELS
+    staged = 8 if padded > 128 else 16
+    return 4 * (3 * staged * padded + 2 * padded + staged * columns * (1 + (groups | 1)))
+
+
+def _recurrence_columns(n_seqs: int, n_heads: int, key_dim: int, value_dim: int) -> int:
+    """Value columns a workgroup of ``decay_recurrence`` takes: as many as its threads (four
+    columns each where that divides) and its LDS hold, fewer where that leaves the chip idle.
+    The results do not depend on it."""
+    groups = (key_dim + RECURRENCE_CHANNELS - 1) // RECURRENCE_CHANNELS
+    most = max(1, min(value_dim, 4 * RECURRENCE_MAX_THREADS // groups, 256))
+    while most > 1 and _recurrence_lds(key_dim, most) > RECURRENCE_MAX_LDS:
+        most -= 1
+    if most >= 8:
+        most -= most % 4
+    elif groups * most > RECURRENCE_MAX_THREADS:
+        most = max(1, RECURRENCE_MAX_THREADS // groups)
     vb = most
-    while vb > 8 and n_seqs * n_heads * ((value_dim + vb - 1) // vb) < RECURRENCE_WORKGROUPS:
-        vb = (vb + 1) // 2
+    # not below what fills a wave with four columns a thread
+    floor = max(8, 4 * 64 // groups // 4 * 4)
+    while vb > floor and n_seqs * n_heads * ((value_dim + vb - 1) // vb) < RECURRENCE_WORKGROUPS:
+        vb = max(floor, vb // 2 // 4 * 4)
     return vb
 
 
