@@ -79,6 +79,8 @@ extern "C" int zf_token_shift_mix(const void* h, int dtype, const float* mu, flo
 #define REC_TC 16          // tokens staged at a time (half of that for more than 128 channels)
 #define REC_MAX_THREADS 256
 #define REC_MAX_LDS 65536
+#define REC_TB 4           // tokens whose partial outputs are summed over the lanes together
+#define REC_STAGE 2        // 8-channel loads a thread has in flight when a chunk comes in
 
 __device__ __forceinline__ float decay_of(float z, int rule, float inv_tau) {
   if (rule == 0) {
@@ -99,14 +101,57 @@ __global__ void decays_in_place_kernel(float* __restrict__ z, const float* __res
   if (i < n) z[i] = decay_of(z[i] + z_bias[i % width], rule, inv_tau);
 }
 
+// 8 neighbouring numbers of a row as floats, through 16-byte loads (the address is a multiple of
+// 16 bytes).
+template <typename T> __device__ __forceinline__ void load8(const T* p, float (&o)[8]);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&o)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&o)[8]) {
+  const uint4 a = *(const uint4*)p;
+  const unsigned w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+// The same in two steps: the bits as they were loaded (a bfloat16 row's 8 numbers take 4
+// registers while they wait), then the floats.
+template <typename T> struct Raw8;
+template <> struct Raw8<float> { float4 a, b; };
+template <> struct Raw8<bf16_t> { uint4 a; };
+__device__ __forceinline__ void load_raw8(const float* p, Raw8<float>& r) {
+  r.a = *(const float4*)p; r.b = *(const float4*)(p + 4);
+}
+__device__ __forceinline__ void load_raw8(const bf16_t* p, Raw8<bf16_t>& r) {
+  r.a = *(const uint4*)p;
+}
+__device__ __forceinline__ void widen8(const Raw8<float>& r, float (&o)[8]) {
+  o[0] = r.a.x; o[1] = r.a.y; o[2] = r.a.z; o[3] = r.a.w;
+  o[4] = r.b.x; o[5] = r.b.y; o[6] = r.b.z; o[7] = r.b.w;
+}
+__device__ __forceinline__ void widen8(const Raw8<bf16_t>& r, float (&o)[8]) {
+  const unsigned w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
 // grid (sequence, head, block of VB value columns); thread (vl, cg) = (tid / CS, tid % CS)
 // holds S[8 cg .. 8 cg + 8, v0 + RV vl .. + RV]: RV value columns (4, 2 or 1: what divides VB),
 // so that a token's q, k and decays, read from LDS once, serve RV columns.  A request's state is
 // laid out [head][dv][CS * 8]: the channels a thread holds lie side by side (channels beyond d
 // are padding that stays zero).  A token's partial outputs (one a thread and column) go to LDS
 // (rows of CS, padded to an odd length so that the sums' reads spread over the banks) and are
-// added in ascending cg, so the sum over channels has one order whatever VB is and however a
-// prompt is cut.
+// added in ascending cg; where CS is a power of two (``shuffle``) the CS lanes of a column add
+// their partial outputs among themselves instead, pair by pair, and lane 0 stores the sum.
+// Either way the sum over channels has one order whatever VB is and however a prompt is cut.  ``wide``: d, dv and VB are multiples of 8 and rows start at multiples of 16
+// bytes; a chunk's rows then come in through 16-byte loads, all of a thread's in flight at once.
 //
 // MODE 0: a sequence's whole portion in one workgroup.  With spans of ``span`` tokens
 // (blockIdx.x = sequence * max_spans + span number): MODE 1 runs a span from a zero state, writes
@@ -122,7 +167,7 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
     float* __restrict__ state, long long slot_stride, const int* __restrict__ state_slots,
     const int* __restrict__ q_start, float* __restrict__ out, int H, int d, int dv, int CS,
     int VB, int TC, int rule, float inv_tau, float q_scale, int span, int max_spans,
-    float* __restrict__ span_state, float* __restrict__ span_decay) {
+    float* __restrict__ span_state, float* __restrict__ span_decay, int wide, int shuffle) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int DP = CS * REC_R;
   const int CSP = CS | 1;
@@ -174,6 +219,59 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
   for (int tc = t0; tc < t1; tc += TC) {
     const int n = min(TC, t1 - tc);
     __syncthreads();                      // the chunk before is read and reduced
+    if (wide && n * CS * 4 >= nthreads) {
+      // a task: 8 channels of a token; REC_STAGE tasks of a thread are in flight at once
+      const int tasks = n * CS;
+      for (int base = 0; base < tasks; base += REC_STAGE * nthreads) {
+        Raw8<T> qr[REC_STAGE], kr[REC_STAGE];
+        Raw8<float> zr[REC_STAGE];
+#pragma unroll
+        for (int u = 0; u < REC_STAGE; ++u) {
+          const int task = base + tid + u * nthreads;
+          if (task < tasks) {
+            const size_t row = (size_t)(tc + task / CS);
+            const int c = hd * d + (task % CS) * 8;
+            if (MODE != 1) load_raw8(q + row * q_stride + c, qr[u]);
+            load_raw8(k + row * k_stride + c, kr[u]);
+            load_raw8(z + row * ((size_t)H * d) + c, zr[u]);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < REC_STAGE; ++u) {
+          const int task = base + tid + u * nthreads;
+          if (task < tasks) {
+            const int at = (task / CS) * DP + (task % CS) * 8;
+            float x8[8];
+            widen8(zr[u], x8);
+            if (rule != 2) {
+              const float* zb = z_bias + hd * d + (task % CS) * 8;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) x8[j] = decay_of(x8[j] + zb[j], rule, inv_tau);
+            }
+            *(float4*)(ds + at) = float4{x8[0], x8[1], x8[2], x8[3]};
+            *(float4*)(ds + at + 4) = float4{x8[4], x8[5], x8[6], x8[7]};
+            widen8(kr[u], x8);
+            *(float4*)(ks + at) = float4{x8[0], x8[1], x8[2], x8[3]};
+            *(float4*)(ks + at + 4) = float4{x8[4], x8[5], x8[6], x8[7]};
+            if (MODE != 1) {
+              widen8(qr[u], x8);
+              *(float4*)(qs + at) = float4{x8[0] * q_scale, x8[1] * q_scale, x8[2] * q_scale,
+                                           x8[3] * q_scale};
+              *(float4*)(qs + at + 4) = float4{x8[4] * q_scale, x8[5] * q_scale, x8[6] * q_scale,
+                                               x8[7] * q_scale};
+            }
+          }
+        }
+      }
+      const int VG = VB / 8;
+      for (int task = tid; task < n * VG; task += nthreads) {
+        const int t = task / VG, x = (task % VG) * 8;
+        float v8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (v0 + x < dv) load8<T>(v + (size_t)(tc + t) * v_stride + hd * dv + v0 + x, v8);
+        *(float4*)(vs + t * VB + x) = float4{v8[0], v8[1], v8[2], v8[3]};
+        *(float4*)(vs + t * VB + x + 4) = float4{v8[4], v8[5], v8[6], v8[7]};
+      }
+    } else {
     for (int i = tid; i < n * DP; i += nthreads) {
       const int t = i / DP, c = i % DP;
       float qv = 0.f, kv = 0.f, dc = 1.f;
@@ -191,6 +289,7 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
       vs[i] = v0 + x < dv ? load_as_float<T>(v + (size_t)(tc + t) * v_stride + hd * dv + v0 + x)
                           : 0.f;
     }
+    }
     __syncthreads();
     if (decays_out)
       for (int c = tid; c < DP; c += nthreads) {
@@ -199,54 +298,97 @@ __global__ __launch_bounds__(REC_MAX_THREADS) void decay_recurrence_kernel(
         pd[c] = p;
       }
     if (active) {
-      for (int t = 0; t < n; ++t) {
-        float vv[RV];
+      float u8[REC_R];
+      if (BEFORE) {
+        const float4* up = (const float4*)(us + cg * REC_R);
+        const float4 u0 = up[0], u1 = up[1];
+        u8[0] = u0.x; u8[1] = u0.y; u8[2] = u0.z; u8[3] = u0.w;
+        u8[4] = u1.x; u8[5] = u1.y; u8[6] = u1.z; u8[7] = u1.w;
+      }
+      // REC_TB tokens at a time, so that their sums over the lanes are in flight together
+      for (int tb = 0; tb < n; tb += REC_TB) {
+        float acc[REC_TB][RV];
 #pragma unroll
-        for (int r = 0; r < RV; ++r) vv[r] = vs[t * VB + col + r];
-        const float4* kp = (const float4*)(ks + t * DP + cg * REC_R);
-        const float4* dp = (const float4*)(ds + t * DP + cg * REC_R);
-        const float4 k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
-        const float k8[REC_R] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-        const float d8[REC_R] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
-        if (MODE == 1) {
+        for (int tt = 0; tt < REC_TB; ++tt) {
 #pragma unroll
-          for (int r = 0; r < RV; ++r)
+          for (int r = 0; r < RV; ++r) acc[tt][r] = 0.f;
+          const int t = tb + tt;
+          if (t >= n) continue;
+          float vv[RV];
 #pragma unroll
-            for (int j = 0; j < REC_R; ++j) S[r][j] = fmaf(d8[j], S[r][j], k8[j] * vv[r]);
-          continue;
-        }
-        const float4* qp = (const float4*)(qs + t * DP + cg * REC_R);
-        const float4 q0 = qp[0], q1 = qp[1];
-        const float q8[REC_R] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-        float u8[REC_R];
-        if (BEFORE) {
-          const float4* up = (const float4*)(us + cg * REC_R);
-          const float4 u0 = up[0], u1 = up[1];
-          u8[0] = u0.x; u8[1] = u0.y; u8[2] = u0.z; u8[3] = u0.w;
-          u8[4] = u1.x; u8[5] = u1.y; u8[6] = u1.z; u8[7] = u1.w;
-        }
+          for (int r = 0; r < RV; ++r) vv[r] = vs[t * VB + col + r];
+          const float4* kp = (const float4*)(ks + t * DP + cg * REC_R);
+          const float4* dp = (const float4*)(ds + t * DP + cg * REC_R);
+          const float4 k0 = kp[0], k1 = kp[1], d0 = dp[0], d1 = dp[1];
+          const float k8[REC_R] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+          const float d8[REC_R] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+          if (MODE == 1) {
 #pragma unroll
-        for (int r = 0; r < RV; ++r) {
-          float acc = 0.f;
-          if (BEFORE) {
+            for (int r = 0; r < RV; ++r)
 #pragma unroll
-            for (int j = 0; j < REC_R; ++j) {
-              const float kv = k8[j] * vv[r];
-              acc = fmaf(q8[j], fmaf(u8[j], kv, S[r][j]), acc);
-              S[r][j] = fmaf(d8[j], S[r][j], kv);
+              for (int j = 0; j < REC_R; ++j) S[r][j] = fmaf(d8[j], S[r][j], k8[j] * vv[r]);
+            continue;
+          }
+          const float4* qp = (const float4*)(qs + t * DP + cg * REC_R);
+          const float4 q0 = qp[0], q1 = qp[1];
+          const float q8[REC_R] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+          for (int r = 0; r < RV; ++r) {
+            float a = 0.f;
+            if (BEFORE) {
+#pragma unroll
+              for (int j = 0; j < REC_R; ++j) {
+                const float kv = k8[j] * vv[r];
+                a = fmaf(q8[j], fmaf(u8[j], kv, S[r][j]), a);
+                S[r][j] = fmaf(d8[j], S[r][j], kv);
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < REC_R; ++j) {
+                S[r][j] = fmaf(d8[j], S[r][j], k8[j] * vv[r]);
+                a = fmaf(q8[j], S[r][j], a);
+              }
             }
-          } else {
+            acc[tt][r] = a;
+          }
+        }
+        if (MODE == 1) continue;
+        if (shuffle) {
+          // CS is a power of two: the CS lanes of a column lie side by side in the wave
+          for (int m = 1; m < CS; m <<= 1) {
 #pragma unroll
-            for (int j = 0; j < REC_R; ++j) {
-              S[r][j] = fmaf(d8[j], S[r][j], k8[j] * vv[r]);
-              acc = fmaf(q8[j], S[r][j], acc);
+            for (int tt = 0; tt < REC_TB; ++tt)
+#pragma unroll
+              for (int r = 0; r < RV; ++r) acc[tt][r] += __shfl_xor(acc[tt][r], m, ZF_WAVE);
+          }
+          // every lane has the sums: lane tt of a column's lanes stores token tt (lane 0 all of
+          // them where there are fewer lanes than tokens)
+#pragma unroll
+          for (int tt = 0; tt < REC_TB; ++tt) {
+            const int t = tb + tt;
+            if (t < n && cg == (CS >= REC_TB ? tt : 0)) {
+              float* o = out + (size_t)(tc + t) * ((size_t)H * dv) + hd * dv + v0 + col;
+              if (RV == 4 && (dv & 3) == 0) {    // a thread's four columns: all within dv or none
+                if (v0 + col < dv)
+                  *(float4*)o = float4{acc[tt][0], acc[tt][1], acc[tt][2], acc[tt][3]};
+              } else {
+#pragma unroll
+                for (int r = 0; r < RV; ++r)
+                  if (v0 + col + r < dv) o[r] = acc[tt][r];
+              }
             }
           }
-          po[(t * VB + col + r) * CSP + cg] = acc;
+        } else {
+#pragma unroll
+          for (int tt = 0; tt < REC_TB; ++tt)
+            if (tb + tt < n) {
+#pragma unroll
+              for (int r = 0; r < RV; ++r) po[((tb + tt) * VB + col + r) * CSP + cg] = acc[tt][r];
+            }
         }
       }
     }
-    if (MODE == 1) continue;
+    if (MODE == 1 || shuffle) continue;
     __syncthreads();
     for (int i = tid; i < n * VB; i += nthreads) {
       const int t = i / VB, x = i % VB;
@@ -300,33 +442,40 @@ __global__ __launch_bounds__(256) void span_states_kernel(
 
 // q, k [T, >= H d], v [T, >= H dv] with contiguous rows (strides in elements), z [T, H d] and
 // out [T, H dv] float32, dense.  CS = ceil(d / 8) <= 32; VB <= 256 value columns a workgroup,
-// RV of them a thread, CS * VB / RV <= 256.
+// RV (1, 2 or 4, dividing VB; another number: the most that divides) of them a thread,
+// CS * VB / RV <= 256.
 extern "C" int zf_decay_recurrence(const void* q, long long q_stride, const void* k,
                                    long long k_stride, const void* v, long long v_stride,
                                    int dtype, const float* z, const float* z_bias,
                                    const float* bonus, float* state, long long slot_stride,
                                    const int* state_slots, const int* q_start, float* out,
-                                   int n_seqs, int H, int d, int dv, int VB, int rule,
+                                   int n_seqs, int H, int d, int dv, int VB, int RV, int rule,
                                    float inv_tau, float q_scale, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   const int CS = (d + REC_R - 1) / REC_R;
-  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 ||
-      CS * (VB / (VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1))) > REC_MAX_THREADS || VB > 256 ||
+  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 || VB > 256 ||
       rule < 0 || rule > 1 || slot_stride < (long long)H * dv * CS * REC_R)
     return -2;
   const int DP = CS * REC_R;
   const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
-  const int RV = VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1);
+  if (RV != 1 && RV != 2 && RV != 4) RV = VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1);
+  if (VB % RV != 0 || CS * (VB / RV) > REC_MAX_THREADS) return -2;
+  const int shuffle = (CS & (CS - 1)) == 0;
   const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + 2 * DP + (size_t)TC * VB +
-                                       (size_t)TC * VB * (CS | 1));
+                                       (shuffle ? 0 : (size_t)TC * VB * (CS | 1)));
   if (smem > REC_MAX_LDS) return -2;
+  const size_t esz = dtype == ZF_F32 ? 4 : 2;
+  const int wide = d % 8 == 0 && dv % 8 == 0 && VB % 8 == 0 && q_stride % 8 == 0 &&
+                   k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
+                   (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 && (uintptr_t)z % 16 == 0 &&
+                   (uintptr_t)z_bias % 16 == 0 && esz > 0;
   const int threads = (CS * (VB / RV) + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
   const dim3 grid(n_seqs, H, (dv + VB - 1) / VB), block(threads);
 #define REC_LAUNCH_RV(TT, BEF, MODE, RVV, GRID, RULE, SPAN, MAXS, SST, SDC)                      \
   hipLaunchKernelGGL((decay_recurrence_kernel<TT, BEF, MODE, RVV>), GRID, block, smem, stream,   \
                      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z,  \
                      z_bias, bonus, state, slot_stride, state_slots, q_start, out, H, d, dv, CS, \
-                     VB, TC, RULE, inv_tau, q_scale, SPAN, MAXS, SST, SDC)
+                     VB, TC, RULE, inv_tau, q_scale, SPAN, MAXS, SST, SDC, wide, shuffle)
 #define REC_LAUNCH(TT, BEF, MODE, GRID, RULE, SPAN, MAXS, SST, SDC)                              \
   if (RV == 4) REC_LAUNCH_RV(TT, BEF, MODE, 4, GRID, RULE, SPAN, MAXS, SST, SDC);                \
   else if (RV == 2) REC_LAUNCH_RV(TT, BEF, MODE, 2, GRID, RULE, SPAN, MAXS, SST, SDC);           \
@@ -352,22 +501,28 @@ extern "C" int zf_decay_recurrence_spans(const void* q, long long q_stride, cons
                                          const float* bonus, float* state, long long slot_stride,
                                          const int* state_slots, const int* q_start, float* out,
                                          int n_tokens, int n_seqs, int H, int d, int dv, int VB,
-                                         int rule, float inv_tau, float q_scale, int span,
+                                         int RV, int rule, float inv_tau, float q_scale, int span,
                                          int max_spans, float* span_state, float* span_decay,
                                          hipStream_t stream) {
   if (n_seqs <= 0 || n_tokens <= 0) return 0;
   const int CS = (d + REC_R - 1) / REC_R;
-  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 ||
-      CS * (VB / (VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1))) > REC_MAX_THREADS || VB > 256 ||
+  if (H <= 0 || d <= 0 || dv <= 0 || CS > 32 || VB < 1 || VB > 256 ||
       rule < 0 || rule > 1 || slot_stride < (long long)H * dv * CS * REC_R || span < REC_TC || span % REC_TC != 0 || max_spans < 1 ||
       span_state == nullptr || span_decay == nullptr)
     return -2;
   const int DP = CS * REC_R;
   const int TC = DP > 128 ? REC_TC / 2 : REC_TC;
-  const int RV = VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1);
+  if (RV != 1 && RV != 2 && RV != 4) RV = VB % 4 == 0 ? 4 : (VB % 2 == 0 ? 2 : 1);
+  if (VB % RV != 0 || CS * (VB / RV) > REC_MAX_THREADS) return -2;
+  const int shuffle = (CS & (CS - 1)) == 0;
   const size_t smem = sizeof(float) * ((size_t)3 * TC * DP + 2 * DP + (size_t)TC * VB +
-                                       (size_t)TC * VB * (CS | 1));
+                                       (shuffle ? 0 : (size_t)TC * VB * (CS | 1)));
   if (smem > REC_MAX_LDS) return -2;
+  const size_t esz = dtype == ZF_F32 ? 4 : 2;
+  const int wide = d % 8 == 0 && dv % 8 == 0 && VB % 8 == 0 && q_stride % 8 == 0 &&
+                   k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
+                   (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 && (uintptr_t)z % 16 == 0 &&
+                   (uintptr_t)z_bias % 16 == 0 && esz > 0;
   const int threads = (CS * (VB / RV) + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
   const dim3 grid(n_seqs * max_spans, H, (dv + VB - 1) / VB), block(threads);
   const long long n = (long long)n_tokens * H * d;

@@ -2370,27 +2370,34 @@ def _recurrence_lds(key_dim: int, columns: int) -> int:
     groups = (key_dim + RECURRENCE_CHANNELS - 1) // RECURRENCE_CHANNELS
     padded = groups * RECURRENCE_CHANNELS
     staged = 8 if padded > 128 else 16
-    return 4 * (3 * staged * padded + 2 * padded + staged * columns * (1 + (groups | 1)))
+    partial = 0 if groups & (groups - 1) == 0 else groups | 1     # none where lanes add them
+    return 4 * (3 * staged * padded + 2 * padded + staged * columns * (1 + partial))
 
 
-def _recurrence_columns(n_seqs: int, n_heads: int, key_dim: int, value_dim: int) -> int:
-    """Value columns a workgroup of ``decay_recurrence`` takes: as many as its threads (four
-    columns each where that divides) and its LDS hold, fewer where that leaves the chip idle.
-    The results do not depend on it."""
+def _recurrence_columns(n_seqs: int, n_heads: int, key_dim: int, value_dim: int,
+                        single: bool = False):
+    """(value columns a workgroup of ``decay_recurrence`` takes, columns a thread).  Portions:
+    four columns a thread where that divides, as many columns as threads and LDS hold, fewer
+    where that leaves the chip idle, though not fewer than fill a wave.  ``single`` (a token a
+    sequence: the state is read and written, little else): a column a thread and small
+    workgroups, so that many loads are in flight.  The results do not depend on either."""
     groups = (key_dim + RECURRENCE_CHANNELS - 1) // RECURRENCE_CHANNELS
-    most = max(1, min(value_dim, 4 * RECURRENCE_MAX_THREADS // groups, 256))
+    per = 1 if single else 4
+    most = max(1, min(value_dim, per * RECURRENCE_MAX_THREADS // groups, 256))
     while most > 1 and _recurrence_lds(key_dim, most) > RECURRENCE_MAX_LDS:
         most -= 1
-    if most >= 8:
-        most -= most % 4
-    elif groups * most > RECURRENCE_MAX_THREADS:
-        most = max(1, RECURRENCE_MAX_THREADS // groups)
+    if single:
+        floor = 8
+    else:
+        if most >= 8:
+            most -= most % 4
+        elif groups * most > RECURRENCE_MAX_THREADS:
+            most = max(1, RECURRENCE_MAX_THREADS // groups)
+        floor = max(8, 4 * 64 // groups // 4 * 4)
     vb = most
-    # not below what fills a wave with four columns a thread
-    floor = max(8, 4 * 64 // groups // 4 * 4)
     while vb > floor and n_seqs * n_heads * ((value_dim + vb - 1) // vb) < RECURRENCE_WORKGROUPS:
-        vb = max(floor, vb // 2 // 4 * 4)
-    return vb
+        vb = max(floor, (vb + 1) // 2 if single else vb // 2 // 4 * 4)
+    return vb, (1 if single else (4 if vb % 4 == 0 else (2 if vb % 2 == 0 else 1)))
 
 
 @_launches("attention")
@@ -2453,7 +2460,7 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
     if span and longest > 2 * span and z.is_contiguous():
         max_spans = (longest + span - 1) // span
         works = n_seqs * max_spans
-        vb = int(columns) if columns is not None else _recurrence_columns(works, H, d, dv)
+        vb, rv = (int(columns), 0) if columns is not None else _recurrence_columns(works, H, d, dv)
         span_state = _workspace("recurrence_span_state", works * need, torch.float32, q.device)
         span_decay = _workspace("recurrence_span_decay", works * (need // dv), torch.float32,
                                 q.device)
@@ -2462,18 +2469,19 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
             ctypes.c_longlong(_columns(k, "decay_recurrence: k")), _ptr(v),
             ctypes.c_longlong(_columns(v, "decay_recurrence: v")), _dt(q), _ptr(z), _ptr(z_bias),
             _ptr(bonus), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(state_slots),
-            _ptr(q_start), _ptr(out), T, n_seqs, H, d, dv, vb, DECAY_RULES[rule],
+            _ptr(q_start), _ptr(out), T, n_seqs, H, d, dv, vb, rv, DECAY_RULES[rule],
             ctypes.c_float(1.0 / tau), ctypes.c_float(q_scale), int(span), max_spans,
             _ptr(span_state), _ptr(span_decay), _stream())
         _check(code, "decay_recurrence_spans")
         return
-    vb = int(columns) if columns is not None else _recurrence_columns(n_seqs, H, d, dv)
+    vb, rv = (int(columns), 0) if columns is not None else \
+        _recurrence_columns(n_seqs, H, d, dv, single=longest == 1)
     code = lib.zf_decay_recurrence(
         _ptr(q), ctypes.c_longlong(_columns(q, "decay_recurrence: q")), _ptr(k),
         ctypes.c_longlong(_columns(k, "decay_recurrence: k")), _ptr(v),
         ctypes.c_longlong(_columns(v, "decay_recurrence: v")), _dt(q), _ptr(z), _ptr(z_bias),
         _ptr(bonus), _ptr(state), ctypes.c_longlong(state.shape[1]), _ptr(state_slots),
-        _ptr(q_start), _ptr(out), n_seqs, H, d, dv, vb, DECAY_RULES[rule],
+        _ptr(q_start), _ptr(out), n_seqs, H, d, dv, vb, rv, DECAY_RULES[rule],
         ctypes.c_float(1.0 / tau), ctypes.c_float(q_scale), _stream())
     _check(code, "decay_recurrence")
 
