@@ -23,6 +23,60 @@
 //  * head_norm_gate      out = o / rms_head(o) * gain * silu(g)
 #include "zf_common.h"
 
+// 8 neighbouring numbers of a row as floats, through 16-byte loads (the address is a multiple of
+// 16 bytes).
+template <typename T> __device__ __forceinline__ void load8(const T* p, float (&o)[8]);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&o)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&o)[8]) {
+  const uint4 a = *(const uint4*)p;
+  const unsigned w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+template <typename T> __device__ __forceinline__ void store8(T* p, const float (&v)[8]);
+template <> __device__ __forceinline__ void store8<float>(float* p, const float (&v)[8]) {
+  *(float4*)p = float4{v[0], v[1], v[2], v[3]};
+  *(float4*)(p + 4) = float4{v[4], v[5], v[6], v[7]};
+}
+template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float (&v)[8]) {
+  unsigned w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = (unsigned)float_to_bf16(v[2 * i]) | ((unsigned)float_to_bf16(v[2 * i + 1]) << 16);
+  *(uint4*)p = uint4{w[0], w[1], w[2], w[3]};
+}
+
+// The same in two steps: the bits as they were loaded (a bfloat16 row's 8 numbers take 4
+// registers while they wait), then the floats.
+template <typename T> struct Raw8;
+template <> struct Raw8<float> { float4 a, b; };
+template <> struct Raw8<bf16_t> { uint4 a; };
+__device__ __forceinline__ void load_raw8(const float* p, Raw8<float>& r) {
+  r.a = *(const float4*)p; r.b = *(const float4*)(p + 4);
+}
+__device__ __forceinline__ void load_raw8(const bf16_t* p, Raw8<bf16_t>& r) {
+  r.a = *(const uint4*)p;
+}
+__device__ __forceinline__ void widen8(const Raw8<float>& r, float (&o)[8]) {
+  o[0] = r.a.x; o[1] = r.a.y; o[2] = r.a.z; o[3] = r.a.w;
+  o[4] = r.b.x; o[5] = r.b.y; o[6] = r.b.z; o[7] = r.b.w;
+}
+__device__ __forceinline__ void widen8(const Raw8<bf16_t>& r, float (&o)[8]) {
+  const unsigned w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
 // ---------------------------------------------------------------- token shift
 // grid (token, block of columns), an element a thread: mixes [n_mix][T][W] in the rows' type.
 // The workgroups of a portion's first token read the state row and are the ones that overwrite
@@ -55,12 +109,66 @@ __global__ void token_shift_mix_kernel(const T* __restrict__ h, const float* __r
   }
 }
 
+// The same with 8 neighbouring columns a thread (W a multiple of 8, rows at multiples of 16
+// bytes): 16-byte loads and stores.  grid (token, block of 8-column groups).
+template <typename T>
+__global__ void token_shift_mix8_kernel(const T* __restrict__ h, const float* __restrict__ mu,
+                                        float* __restrict__ state, long long slot_stride,
+                                        const int* __restrict__ state_slots,
+                                        const int* __restrict__ seq_index,
+                                        const int* __restrict__ q_start, T* __restrict__ out,
+                                        int n_tokens, int W, int n_mix) {
+  const int t = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= W) return;
+  const int s = seq_index[t];
+  const int t0 = q_start[s], t1 = q_start[s + 1];
+  const bool first = t == t0;
+  const T* row = h + (size_t)t * W;
+  float* st = state + (size_t)state_slots[s] * slot_stride;
+  float x[8], p[8];
+  load8<T>(row + i, x);
+  if (first) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p[j] = st[i + j];
+  } else {
+    load8<T>(row - W + i, p);
+  }
+  for (int m = 0; m < n_mix; ++m) {
+    float g[8], y[8];
+    load8<float>(mu + (size_t)m * W + i, g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = fmaf(p[j] - x[j], g[j], x[j]);
+    store8<T>(out + ((size_t)m * n_tokens + t) * W + i, y);
+  }
+  if (first) {
+    float l[8];
+    load8<T>(h + (size_t)(t1 - 1) * W + i, l);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) st[i + j] = l[j];
+  }
+}
+
 extern "C" int zf_token_shift_mix(const void* h, int dtype, const float* mu, float* state,
                                   long long slot_stride, const int* state_slots,
                                   const int* seq_index, const int* q_start, void* out, int T,
                                   int W, int n_mix, hipStream_t stream) {
   if (T <= 0) return 0;
   if (W <= 0 || n_mix <= 0) return -2;
+  if (W % 8 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)mu % 16 == 0) {
+    const int groups = W / 8;
+    const int block = groups >= 256 ? 256 : (groups + ZF_WAVE - 1) / ZF_WAVE * ZF_WAVE;
+    const dim3 grid(T, (groups + block - 1) / block);
+    if (dtype == ZF_F32)
+      hipLaunchKernelGGL(token_shift_mix8_kernel<float>, grid, dim3(block), 0, stream,
+                         (const float*)h, mu, state, slot_stride, state_slots, seq_index, q_start,
+                         (float*)out, T, W, n_mix);
+    else
+      hipLaunchKernelGGL(token_shift_mix8_kernel<bf16_t>, grid, dim3(block), 0, stream,
+                         (const bf16_t*)h, mu, state, slot_stride, state_slots, seq_index,
+                         q_start, (bf16_t*)out, T, W, n_mix);
+    ZF_CHECK_LAUNCH();
+  }
   const int block = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
   const dim3 grid(T, (W + block - 1) / block);
   if (dtype == ZF_F32)
@@ -99,47 +207,6 @@ __global__ void decays_in_place_kernel(float* __restrict__ z, const float* __res
                                        long long n, int width, int rule, float inv_tau) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) z[i] = decay_of(z[i] + z_bias[i % width], rule, inv_tau);
-}
-
-// 8 neighbouring numbers of a row as floats, through 16-byte loads (the address is a multiple of
-// 16 bytes).
-template <typename T> __device__ __forceinline__ void load8(const T* p, float (&o)[8]);
-template <> __device__ __forceinline__ void load8<float>(const float* p, float (&o)[8]) {
-  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
-  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
-}
-template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&o)[8]) {
-  const uint4 a = *(const uint4*)p;
-  const unsigned w[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    o[2 * i] = __uint_as_float(w[i] << 16);
-    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-  }
-}
-
-// The same in two steps: the bits as they were loaded (a bfloat16 row's 8 numbers take 4
-// registers while they wait), then the floats.
-template <typename T> struct Raw8;
-template <> struct Raw8<float> { float4 a, b; };
-template <> struct Raw8<bf16_t> { uint4 a; };
-__device__ __forceinline__ void load_raw8(const float* p, Raw8<float>& r) {
-  r.a = *(const float4*)p; r.b = *(const float4*)(p + 4);
-}
-__device__ __forceinline__ void load_raw8(const bf16_t* p, Raw8<bf16_t>& r) {
-  r.a = *(const uint4*)p;
-}
-__device__ __forceinline__ void widen8(const Raw8<float>& r, float (&o)[8]) {
-  o[0] = r.a.x; o[1] = r.a.y; o[2] = r.a.z; o[3] = r.a.w;
-  o[4] = r.b.x; o[5] = r.b.y; o[6] = r.b.z; o[7] = r.b.w;
-}
-__device__ __forceinline__ void widen8(const Raw8<bf16_t>& r, float (&o)[8]) {
-  const unsigned w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    o[2 * i] = __uint_as_float(w[i] << 16);
-    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-  }
 }
 
 // grid (sequence, head, block of VB value columns); thread (vl, cg) = (tid / CS, tid % CS)
