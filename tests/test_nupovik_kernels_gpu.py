@@ -213,6 +213,8 @@ SPANNED = [  # H, d, dv, rule, bonus, tau, span, lens of the first step, lens of
     (2, 136, 8, "double_exp", True, 1.0, 16, [48, 50], [35, 1]),
     (4, 8, 16, "double_exp", True, 1.0, None, [300, 129, 5], [130, 1, 260]),
     (1, 7, 3, "sigmoid_root", True, 2.5, 48, [150], [97]),
+    # more tokens than the most spans of the usual length hold: the spans grow
+    (1, 8, 4, "sigmoid_root", False, 8.0, None, [4200, 70], [3, 1]),
 ]
 
 
