@@ -77,7 +77,8 @@ class KVGroup:
 
 class CacheManager:
     """``needs[pos]`` is the cache need of schedule position ``pos`` (None: no cache of its
-    own); ``reads[pos]`` names the position whose cache a run reads instead.  The pools are
+    own; a tuple: one ``KVNeed`` and one ``StateNeed``, and the run's view holds both);
+    ``reads[pos]`` names the position whose cache a run reads instead.  The pools are
     tensors of this class; which pages are free, the block tables and the slots are kept by
     the native core, where a request goes by a number that this class gives it."""
 
@@ -94,13 +95,20 @@ class CacheManager:
         by_need: Dict[KVNeed, List[int]] = {}
         self.state_pools: Dict[int, torch.Tensor] = {}
         for pos, need in enumerate(needs):
-            if isinstance(need, KVNeed):
-                by_need.setdefault(need, []).append(pos)
-            elif isinstance(need, StateNeed):
-                self.state_pools[pos] = torch.zeros((max_requests,) + tuple(need.shape),
-                                                    dtype=need.dtype, device=device)
-            elif need is not None:
-                raise StepError(f"unknown cache need {need!r}")
+            # a run may bring both kinds (two mixers side by side): a tuple with one of each
+            both = tuple(need) if isinstance(need, (tuple, list)) else (need,)
+            if sum(isinstance(n, KVNeed) for n in both) > 1 \
+                    or sum(isinstance(n, StateNeed) for n in both) > 1:
+                raise StepError(f"run {pos} asks for more than one cache of keys and values or "
+                                f"more than one state: {need!r}")
+            for one in both:
+                if isinstance(one, KVNeed):
+                    by_need.setdefault(one, []).append(pos)
+                elif isinstance(one, StateNeed):
+                    self.state_pools[pos] = torch.zeros((max_requests,) + tuple(one.shape),
+                                                        dtype=one.dtype, device=device)
+                elif one is not None:
+                    raise StepError(f"unknown cache need {one!r}")
         self._lib = core_lib()
         windows = [-1 if need.window is None else int(need.window) for need in by_need]
         self._core = ctypes.c_void_p(self._lib.zc_create(

@@ -13,3 +13,5 @@ from .qwen3 import Qwen3Config
 from .fezupel import FezupelConfig
 from .lodenex import LodenexConfig
 from .nupovik import NupovikConfig
+from .specs import GatedDeltaRuleSpec, ParallelMixerSpec, StreamBlockSpec
+from .kugisun import KugisunConfig

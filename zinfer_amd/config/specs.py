@@ -29,6 +29,7 @@ class LayerNormSpec:
     centred: bool = True
     weight_name: str = "weight"
     bias_name: Optional[str] = "bias"
+    gain_offset: float = 0.0               # the gain is this plus the stored weight
 
 
 @dataclass(frozen=True)
@@ -87,10 +88,12 @@ class LeadingRotarySpec:
     ``magnitude``.  The frequencies are plain data, so that any rule for them (a base alone,
     wavelengths slowed beyond a length, a ramp between two turn counts) gives the same part;
     ``config.rotary`` holds the rules.  There is no table of positions: the angle is formed
-    from the position where it is used, in 32-bit."""
+    from the position where it is used, in 32-bit.  ``interleaved``: the pairs are the
+    neighbours (2i, 2i + 1) instead, pair i turning by frequencies[i]."""
     dims: int
     frequencies: Tuple[float, ...]
     magnitude: float = 1.0
+    interleaved: bool = False
 
 
 @dataclass(frozen=True)
@@ -102,8 +105,10 @@ class MaskedGqaAttentionSpec:
     ``window`` (the last ``window`` positions) and ``chunk`` (only keys of the query's own
     chunk of that many positions, counted from position 0); ``sink``: one learned number a head
     whose exponential joins the soft-max's denominator; ``head_gate``: head h's output is
-    multiplied by sigmoid(W_g h)_h, one number a head.  The ``*_name`` fields are the tensor
-    names below the mixer's prefix."""
+    multiplied by sigmoid(W_g h)_h, one number a head.  ``qk_norm_per_head``: the norm of q and
+    of k runs over every head on its own instead, with one gain of ``head_dim`` for all heads.
+    ``bias``: q, k and v have biases (``bias_suffix`` behind the matrix's name), added before
+    the norm.  The ``*_name`` fields are the tensor names below the mixer's prefix."""
     hidden_size: int
     n_heads: int
     n_kv_heads: int
@@ -111,6 +116,9 @@ class MaskedGqaAttentionSpec:
     value_dim: int
     scale: float
     qk_norm_eps: Optional[float] = None
+    qk_norm_per_head: bool = False
+    bias: bool = False
+    bias_suffix: str = ".b"
     rotary: Optional[LeadingRotarySpec] = None
     softcap: Optional[float] = None
     window: Optional[int] = None
@@ -233,6 +241,55 @@ class TokenShiftRecurrenceSpec:
 
 
 @dataclass(frozen=True)
+class GatedDeltaRuleSpec:
+    """A mixer whose memory is one matrix a head, S [head_dim, value_dim], carried from token to
+    token in 32-bit and corrected towards every token's value: S <- g_t S; w = beta_t (v_t -
+    S^T k_t); S <- S + k_t w^T; o_t = S^T q_t.  q and k (``n_kv_heads`` heads of ``head_dim``)
+    and v (``n_heads`` heads of ``value_dim``; value head n reads q/k head floor(n / (n_heads /
+    n_kv_heads))) each pass a causal convolution over time a channel (``conv_taps`` taps, the
+    last one the token's own, zeros before a sequence's start; the taps - 1 rows before a step
+    are part of the state) and silu; q and k then become unit vectors a head, x / sqrt(sum x^2 +
+    ``unit_eps``), and q is multiplied by ``q_scale`` (None: head_dim^(-1/2)).  One decay and one
+    step size a head and token: g = exp(-exp(A) softplus(W_a h + dt)), beta = sigmoid(W_b h).
+    Each head's o goes through an RMS norm over value_dim with one gain for all heads, the heads
+    side by side are multiplied by silu(W_g h), then W_o.  The ``*_name`` fields are the tensor
+    names below the mixer's prefix (``conv_suffix`` behind a matrix's name: its taps)."""
+    hidden_size: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    conv_taps: int
+    norm_eps: float
+    unit_eps: float = 1e-6
+    q_scale: Optional[float] = None
+    q_name: str = "q"
+    k_name: str = "k"
+    v_name: str = "v"
+    conv_suffix: str = ".conv"
+    beta_name: str = "b"
+    decay_name: str = "a"
+    decay_log_name: str = "A_log"
+    decay_bias_name: str = "dt_bias"
+    gate_name: str = "g"
+    norm_name: str = "norm"
+    o_name: str = "o"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers side by side that read the same input: ``left_scale`` * left(h) +
+    ``right_scale`` * right(h).  Each has its own tensors (below ``left_prefix`` and
+    ``right_prefix``) and its own cache or state."""
+    left: object
+    right: object
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    left_prefix: str = "left."
+    right_prefix: str = "right."
+
+
+@dataclass(frozen=True)
 class PlainExpertSpec:
     """down(act(up(x))), no gate and no bias; ``activation`` as in ``DenseMlpSpec``."""
     intermediate_size: int
@@ -259,6 +316,14 @@ class MoeSpec:
     weights are the chosen experts' s over their sum (+ 1e-20); with ``groups`` = (count, keep)
     the experts form ``count`` equal groups of neighbours, a group is marked by the sum of its
     two largest choice scores, and only experts of the ``keep`` best groups can be chosen.
+    ``scoring`` "softmax_all": as "sigmoid" with s = softmax(z) over all the router's outputs.
+    ``group_mark``: how many of a group's largest choice scores make its mark (2 or 1).
+    ``normalize`` False: the weights are the chosen s themselves; either way they are
+    multiplied by ``weight_scale``.  ``n_identity``: the router has that many outputs more
+    than there are experts; one of them, chosen, stands for an expert without tensors whose
+    output is its input (times the weight); they count as experts in groups and choice.
+    ``shared_gate_name``: the shared expert's output is multiplied by sigmoid(w . x), one
+    number a token, w being that tensor [1, hidden] below ``shared_prefix``.
     ``expert`` is a ``GatedExpertSpec`` or a ``PlainExpertSpec`` (no gate matrix).  Tensor names
     below the part's prefix: the router's matrix and bias, ``expert_prefix.format(e)`` and
     ``shared_prefix`` followed by the matrices' names."""
@@ -271,6 +336,11 @@ class MoeSpec:
     scoring: str = "softmax"
     correction_name: Optional[str] = None
     groups: Optional[Tuple[int, int]] = None
+    group_mark: int = 2
+    normalize: bool = True
+    weight_scale: float = 1.0
+    n_identity: int = 0
+    shared_gate_name: Optional[str] = None
     router_name: str = "gate.weight"
     router_bias_name: str = "gate.bias"
     expert_prefix: str = "experts.{}."
@@ -282,9 +352,13 @@ class MoeSpec:
 
 @dataclass(frozen=True)
 class SwiGluSpec:
-    """down(silu(gate(x)) * up(x))."""
+    """down(silu(gate(x)) * up(x)); the ``*_name`` fields are the tensor names below the
+    part's prefix."""
     hidden_size: int
     intermediate_size: int
+    gate_name: str = "gate_proj.weight"
+    up_name: str = "up_proj.weight"
+    down_name: str = "down_proj.weight"
 
 
 @dataclass(frozen=True)
@@ -351,6 +425,31 @@ class ParallelBlockSpec:
 
 
 @dataclass(frozen=True)
+class StreamBlockSpec:
+    """A layer over ``streams`` copies X_1 .. X_S of the residual stream instead of one.  For
+    each sublayer c (the mixer, then the feed-forward if there is one): u = sum_s a_c[s] X_s;
+    y = sublayer_c(norm_c(u)); X_t <- sum_s M_c[s, t] X_s + b_c[t] y for all t at once from the
+    old X.  a_c [S], M_c [S, S] (indexed [from, to]) and b_c [S] are the tensors
+    ``coef_prefix.format(c) + in_name | mix_name | out_name`` below the layer's prefix;
+    ``learned`` False: there are no such tensors, a = b = 1 and M the identity (with one
+    stream that is the plain pre-norm layer x += sublayer(norm(x)))."""
+    streams: int
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_norm: object
+    ff_norm: Optional[object] = None
+    learned: bool = True
+    mixer_prefix: str = "mix."
+    ff_prefix: str = "mlp."
+    mixer_norm_prefix: str = "norm1"
+    ff_norm_prefix: str = "norm2"
+    coef_prefix: str = "hc{}."
+    in_name: str = "in"
+    mix_name: str = "mix"
+    out_name: str = "out"
+
+
+@dataclass(frozen=True)
 class SinusoidalPositionSpec:
     """A position vector added to the embedding row, formed from the position where it is used:
     entry 2i is sin(p * f_i), entry 2i + 1 cos(p * f_i), f_i = base^(-2i / width)."""
@@ -396,3 +495,10 @@ class ModelSpec:
     sinusoidal_positions: Optional[SinusoidalPositionSpec] = None
     # the matrix [hidden, 2 hidden] of the schedule entries that say ``reentry``
     reentry_name: Optional[str] = None
+    # the residual stream in that many copies [streams, T, hidden], all equal to the embedding's
+    # output at the start and added up before the final norm (the blocks are ``StreamBlockSpec``
+    # layers); None: the one stream [T, hidden]
+    streams: Optional[int] = None
+    # the number each of ``layers`` goes by in ``layer_prefix`` (None: its index): a model whose
+    # file numbers all runs while some of them bring no tensors of their own
+    layer_numbers: Optional[Tuple[int, ...]] = None

@@ -16,10 +16,10 @@
 // been moved to the query's and the output's side (one kv head, a key row = the latent and the
 // rotated part, the value = the latent).
 //
-//  * project_rows: the rows of a projection, segment by segment: an RMS norm over the whole
-//    segment, a rotation of some leading elements of every head by the token's position
-//    (angle = position * frequency in 32-bit, pairs (i, i + dims / 2)), then to plain rows or
-//    into the pools at slot_mapping.
+//  * project_rows: the rows of a projection, segment by segment: a bias, an RMS norm over the
+//    whole segment or over every head on its own, a rotation of some leading elements of every
+//    head by the token's position (angle = position * frequency in 32-bit, pairs (i, i + dims /
+//    2) or neighbours (2i, 2i + 1)), then to plain rows or into the pools at slot_mapping.
 //  * masked_attention: any sizes, both dtypes, all arithmetic 32-bit; one workgroup a (token,
 //    kv head), one wave a query head.  A token's chunks of keys start at the first key it sees,
 //    so its result never depends on how the batch was cut.
@@ -41,6 +41,9 @@ __host__ __device__ __forceinline__ size_t pool_at(int r, int d, int page_size, 
 struct RowSegment {
   int src_off, width;        // columns [src_off, src_off + width) of a source row
   const float* gain;         // [width]: RMS norm over the whole segment; null: none
+  const float* bias;         // [width], added to the source's values first; null: none
+  int per_head;              // the norm runs over every head alone, gain [hd] for all heads
+  int interleaved;           // the rotated pairs are neighbours (2i, 2i + 1), pair i by freq[i]
   float eps;
   int hd;                    // head size inside the segment (width % hd == 0)
   int rot_off, rot_dims;     // elements [rot_off, rot_off + rot_dims) of a head are rotated
@@ -60,6 +63,7 @@ struct RowSegments {
 };
 
 #define PR_MAX_PAIRS 256      // a rotation's cosines and sines are kept in LDS: rot_dims <= 512
+#define PR_MAX_HEADS 256      // a norm a head keeps the heads' factors in LDS
 
 template <typename T>
 __global__ __launch_bounds__(256) void project_rows_kernel(
@@ -68,6 +72,7 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
 #pragma clang fp contract(off)
   __shared__ float red[16];
   __shared__ float cs_t[PR_MAX_PAIRS], sn_t[PR_MAX_PAIRS];
+  __shared__ float inv_h[PR_MAX_HEADS];
   const int t = blockIdx.x;
   const T* row = src + (size_t)t * src_stride;
   const float pos = (float)positions[t];
@@ -77,14 +82,30 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
     const RowSegment& g = segs.s[si];
     const T* x = row + g.src_off;
     float inv = 1.f;
-    if (g.gain != nullptr) {
+    if (g.gain != nullptr && !g.per_head) {
       float ss = 0.f;
       for (int i = threadIdx.x; i < g.width; i += blockDim.x) {
-        const float v = load_as_float<T>(x + i);
+        float v = load_as_float<T>(x + i);
+        if (g.bias != nullptr) v = v + g.bias[i];
         ss += v * v;
       }
       ss = block_sum(ss, red);
       inv = 1.0f / sqrtf(ss / (float)g.width + g.eps);
+    } else if (g.gain != nullptr) {
+      // a wave a head: lanes side by side over its elements, then over the lanes
+      __syncthreads();                               // the segment before is done with inv_h
+      const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
+      for (int head = wave; head < g.width / g.hd; head += blockDim.x / ZF_WAVE) {
+        float ss = 0.f;
+        for (int d = lane; d < g.hd; d += ZF_WAVE) {
+          float v = load_as_float<T>(x + head * g.hd + d);
+          if (g.bias != nullptr) v = v + g.bias[head * g.hd + d];
+          ss += v * v;
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) inv_h[head] = 1.0f / sqrtf(ss / (float)g.hd + g.eps);
+      }
+      __syncthreads();
     }
     size_t pool_base = 0;
     int pool_row = 0;
@@ -113,14 +134,18 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
       const int head = i / g.hd, d = i % g.hd;
       if (d < g.skip) continue;
       float a = load_as_float<T>(x + i);
-      if (g.gain != nullptr) a = a * inv * g.gain[i];
+      if (g.bias != nullptr) a = a + g.bias[i];
+      const float inv_i = g.per_head ? inv_h[head] : inv;
+      if (g.gain != nullptr) a = a * inv_i * g.gain[g.per_head ? d : i];
       const int r = d - g.rot_off;
       if (r >= 0 && r < g.rot_dims) {
-        const bool first = r < half;
-        const int pi = first ? i + half : i - half;
+        const bool first = g.interleaved ? (r & 1) == 0 : r < half;
+        const int step = g.interleaved ? 1 : half;
+        const int pi = first ? i + step : i - step;
         float b = load_as_float<T>(x + pi);
-        if (g.gain != nullptr) b = b * inv * g.gain[pi];
-        const int j = first ? r : r - half;
+        if (g.bias != nullptr) b = b + g.bias[pi];
+        if (g.gain != nullptr) b = b * inv_i * g.gain[g.per_head ? pi - head * g.hd : pi];
+        const int j = g.interleaved ? r >> 1 : (first ? r : r - half);
         const float cs = cs_t[j], sn = sn_t[j];
         a = first ? a * cs - b * sn : a * cs + b * sn;
       }
@@ -151,12 +176,25 @@ __device__ __forceinline__ void pr_unpack8(const uint4& v, float (&f)[8]) {
   }
 }
 
+// 8 elements of a row from column i on, with the bias (if any) added
+__device__ __forceinline__ void pr_load8(const bf16_t* x, const float* bias, int i, float (&f)[8]) {
+#pragma clang fp contract(off)
+  pr_unpack8(*(const uint4*)(x + i), f);
+  if (bias != nullptr) {
+    const float4 b0 = *(const float4*)(bias + i), b1 = *(const float4*)(bias + i + 4);
+    const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = f[e] + bb[e];
+  }
+}
+
 __global__ __launch_bounds__(256) void project_rows_vec8_kernel(
     const bf16_t* __restrict__ src, long long src_stride, const int* __restrict__ positions,
     const int* __restrict__ slot_mapping, int page_size, RowSegments segs) {
 #pragma clang fp contract(off)
   __shared__ float red[16];
   __shared__ float cs_t[PR_MAX_PAIRS], sn_t[PR_MAX_PAIRS];
+  __shared__ float inv_h[PR_MAX_HEADS];
   const int t = blockIdx.x;
   const bf16_t* row = src + (size_t)t * src_stride;
   const float pos = (float)positions[t];
@@ -167,16 +205,31 @@ __global__ __launch_bounds__(256) void project_rows_vec8_kernel(
     const bf16_t* x = row + g.src_off;
     const int n8 = g.width / 8;
     float inv = 1.f;
-    if (g.gain != nullptr) {
+    if (g.gain != nullptr && !g.per_head) {
       float ss = 0.f;
       for (int c = threadIdx.x; c < n8; c += blockDim.x) {
         float f[8];
-        pr_unpack8(*(const uint4*)(x + 8 * c), f);
+        pr_load8(x, g.bias, 8 * c, f);
 #pragma unroll
         for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
       }
       ss = block_sum(ss, red);
       inv = 1.0f / sqrtf(ss / (float)g.width + g.eps);
+    } else if (g.gain != nullptr) {
+      __syncthreads();
+      const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
+      for (int head = wave; head < g.width / g.hd; head += blockDim.x / ZF_WAVE) {
+        float ss = 0.f;
+        for (int c = lane; c < g.hd / 8; c += ZF_WAVE) {
+          float f[8];
+          pr_load8(x, g.bias, head * g.hd + 8 * c, f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) inv_h[head] = 1.0f / sqrtf(ss / (float)g.hd + g.eps);
+      }
+      __syncthreads();
     }
     size_t pool_base = 0;
     int pool_row = 0;
@@ -204,24 +257,38 @@ __global__ __launch_bounds__(256) void project_rows_vec8_kernel(
       const int head = i / g.hd, d = i % g.hd;
       if (d < g.skip) continue;
       float a[8];
-      pr_unpack8(*(const uint4*)(x + i), a);
+      pr_load8(x, g.bias, i, a);
+      const float inv_i = g.per_head ? inv_h[head] : inv;
       if (g.gain != nullptr) {
-        const float4 g0 = *(const float4*)(g.gain + i), g1 = *(const float4*)(g.gain + i + 4);
+        const int gi = g.per_head ? d : i;
+        const float4 g0 = *(const float4*)(g.gain + gi), g1 = *(const float4*)(g.gain + gi + 4);
         const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) a[e] = a[e] * inv * gg[e];
+        for (int e = 0; e < 8; ++e) a[e] = a[e] * inv_i * gg[e];
       }
       const int r = d - g.rot_off;
-      if (r >= 0 && r < g.rot_dims) {
+      if (r >= 0 && r < g.rot_dims && g.interleaved) {
+        // the partner of an element is its neighbour, among the same 8
+        float n[8];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const float cs = cs_t[(r + e) >> 1], sn = sn_t[(r + e) >> 1];
+          n[e] = a[e] * cs - a[e + 1] * sn;
+          n[e + 1] = a[e + 1] * cs + a[e] * sn;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] = n[e];
+      } else if (r >= 0 && r < g.rot_dims) {
         const bool first = r < half;
         const int pi = first ? i + half : i - half;
         float b[8];
-        pr_unpack8(*(const uint4*)(x + pi), b);
+        pr_load8(x, g.bias, pi, b);
         if (g.gain != nullptr) {
-          const float4 g0 = *(const float4*)(g.gain + pi), g1 = *(const float4*)(g.gain + pi + 4);
+          const int gi = g.per_head ? pi - head * g.hd : pi;
+          const float4 g0 = *(const float4*)(g.gain + gi), g1 = *(const float4*)(g.gain + gi + 4);
           const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
-          for (int e = 0; e < 8; ++e) b[e] = b[e] * inv * gg[e];
+          for (int e = 0; e < 8; ++e) b[e] = b[e] * inv_i * gg[e];
         }
         const int j = first ? r : r - half;
 #pragma unroll
@@ -244,8 +311,8 @@ __global__ __launch_bounds__(256) void project_rows_vec8_kernel(
 }
 
 // ints: 11 a segment (src_off, width, hd, rot_off, rot_dims, skip, to_pool, dst_off, dst_hd,
-// pool_heads, 0); floats: 2 a segment (eps, mag); ptrs: 3 a segment (gain, freq, dst);
-// strides: 1 a segment
+// pool_heads, flags: 1 = a norm a head, 2 = neighbouring pairs); floats: 2 a segment (eps, mag);
+// ptrs: 4 a segment (gain, freq, dst, bias); strides: 1 a segment
 extern "C" int zf_project_rows(const void* src, int dtype, long long src_stride,
                                const int* positions, const int* slot_mapping, int T,
                                int page_size, int n_segs, const int* ints, const float* floats,
@@ -260,9 +327,11 @@ extern "C" int zf_project_rows(const void* src, int dtype, long long src_stride,
     g.src_off = v[0]; g.width = v[1]; g.hd = v[2]; g.rot_off = v[3]; g.rot_dims = v[4];
     g.skip = v[5]; g.to_pool = v[6]; g.dst_off = v[7]; g.dst_hd = v[8]; g.pool_heads = v[9];
     g.eps = floats[2 * i]; g.mag = floats[2 * i + 1];
-    g.gain = (const float*)ptrs[3 * i]; g.freq = (const float*)ptrs[3 * i + 1];
-    g.dst = ptrs[3 * i + 2];
+    g.per_head = v[10] & 1; g.interleaved = (v[10] >> 1) & 1;
+    g.gain = (const float*)ptrs[4 * i]; g.freq = (const float*)ptrs[4 * i + 1];
+    g.dst = ptrs[4 * i + 2]; g.bias = (const float*)ptrs[4 * i + 3];
     g.dst_stride = strides[i];
+    if (g.per_head && g.gain != nullptr && g.hd > 0 && g.width / g.hd > PR_MAX_HEADS) return -2;
     if (g.width <= 0 || g.hd <= 0 || g.width % g.hd != 0 || g.rot_dims < 0 || g.rot_dims % 2 != 0
         || g.rot_off < 0 || g.rot_off + g.rot_dims > g.hd || g.skip < 0 || g.skip >= g.hd
         || (g.rot_dims > 0 && g.freq == nullptr) || g.rot_dims > 2 * PR_MAX_PAIRS
@@ -273,7 +342,9 @@ extern "C" int zf_project_rows(const void* src, int dtype, long long src_stride,
   bool vec8 = dtype == ZF_BF16 && src_stride % 8 == 0 && (uintptr_t)src % 16 == 0;
   for (int i = 0; i < n_segs && vec8; ++i) {
     const RowSegment& g = segs.s[i];
-    vec8 = g.src_off % 8 == 0 && g.hd % 8 == 0 && g.rot_off % 8 == 0 && g.rot_dims % 16 == 0
+    vec8 = g.src_off % 8 == 0 && g.hd % 8 == 0 && g.rot_off % 8 == 0
+        && g.rot_dims % (g.interleaved ? 8 : 16) == 0
+        && (g.bias == nullptr || (uintptr_t)g.bias % 16 == 0)
         && g.skip % 8 == 0 && g.dst_off % 8 == 0 && g.dst_hd % 8 == 0 && (uintptr_t)g.dst % 16 == 0
         && (g.to_pool || g.dst_stride % 8 == 0) && (g.gain == nullptr || (uintptr_t)g.gain % 16 == 0);
   }

@@ -53,7 +53,8 @@ template <typename T>
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ router, const float* __restrict__ bias,
     int* __restrict__ ids, float* __restrict__ weights, int n_tokens, int W, int E, int top,
-    int scoring, const float* __restrict__ correction, int n_groups, int keep_groups) {
+    int scoring, const float* __restrict__ correction, int n_groups, int keep_groups,
+    int mark_top, int normalize, float weight_scale, int n_extra, float* __restrict__ extra) {
   __shared__ float zs[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS], shares[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
   __shared__ int chosens[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
   __shared__ unsigned char kepts[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
@@ -62,7 +63,8 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
   const T* rows[MOE_ROUTE_TOKENS];
 #pragma unroll
   for (int k = 0; k < MOE_ROUTE_TOKENS; ++k) rows[k] = h + (size_t)min(t0 + k, n_tokens - 1) * W;
-  for (int e = wave; e < E; e += MOE_ROUTE_WAVES) {
+  // (rows E .. E + n_extra - 1 of the router are no experts: their sigmoids go to `extra`)
+  for (int e = wave; e < E + n_extra; e += MOE_ROUTE_WAVES) {
     const float* r = router + (size_t)e * W;
     float dot[MOE_ROUTE_TOKENS];
 #pragma unroll
@@ -89,11 +91,15 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
           dot[k] = fmaf(load_as_float<T>(rows[k] + i), rv, dot[k]);
       }
     }
-    const float be = bias != nullptr ? bias[e] : 0.f;
+    const float be = (bias != nullptr && e < E) ? bias[e] : 0.f;
 #pragma unroll
     for (int k = 0; k < MOE_ROUTE_TOKENS; ++k) {
       const float z = wave_sum(dot[k]);
-      if (lane == 0) zs[k][e] = z + be;
+      if (lane == 0) {
+        if (e < E) zs[k][e] = z + be;
+        else if (t0 + k < n_tokens)
+          extra[(size_t)(t0 + k) * n_extra + (e - E)] = 1.0f / (1.0f + expf(-z));
+      }
     }
   }
   __syncthreads();
@@ -102,10 +108,20 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
   float* z = zs[wave];
   float* share = shares[wave];
   int* chosen = chosens[wave];
-  if (scoring == 1) {
-    // scores s = sigmoid(z) (kept in `share`), choice scores s + correction (in `z`)
+  if (scoring != 0) {
+    // scores s = sigmoid(z), or the soft-max over all of z (kept in `share`), choice scores
+    // s + correction (in `z`)
+    float zmax = 0.f, zsum = 1.f;
+    if (scoring == 2) {
+      zmax = -INFINITY;
+      for (int e = lane; e < E; e += ZF_WAVE) zmax = fmaxf(zmax, z[e]);
+      zmax = wave_max(zmax);
+      zsum = 0.f;
+      for (int e = lane; e < E; e += ZF_WAVE) zsum += expf(z[e] - zmax);
+      zsum = wave_sum(zsum);
+    }
     for (int e = lane; e < E; e += ZF_WAVE) {
-      const float sc = 1.0f / (1.0f + expf(-z[e]));
+      const float sc = scoring == 2 ? expf(z[e] - zmax) / zsum : 1.0f / (1.0f + expf(-z[e]));
       share[e] = sc;
       z[e] = sc + (correction != nullptr ? correction[e] : 0.f);
     }
@@ -122,7 +138,7 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
           const float v = z[e];
           if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
         }
-        mark[g] = size > 1 ? a + b : a;
+        mark[g] = (size > 1 && mark_top > 1) ? a + b : a;
         kept[g] = 0;
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -177,7 +193,8 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
     }
     for (int k = lane; k < top; k += ZF_WAVE) {
       ids[(size_t)t * top + k] = chosen[k];
-      weights[(size_t)t * top + k] = share[chosen[k]] / (sum + 1e-20f);
+      const float sh = share[chosen[k]];
+      weights[(size_t)t * top + k] = (normalize ? sh / (sum + 1e-20f) : sh) * weight_scale;
     }
     return;
   }
@@ -217,9 +234,11 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
 extern "C" int zf_moe_route(const void* h, int dtype, const float* router, const float* bias,
                             int* ids, float* weights, int T, int W, int E, int top,
                             int scoring, const float* correction, int n_groups, int keep_groups,
-                            hipStream_t stream) {
+                            int mark_top, int normalize, float weight_scale, int n_extra,
+                            float* extra, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E || scoring < 0 || scoring > 1 ||
+  if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E || scoring < 0 || scoring > 2 ||
+      n_extra < 0 || (n_extra > 0 && extra == nullptr) || mark_top < 1 || mark_top > 2 ||
       n_groups < 0 || (n_groups > 0 && (E % n_groups != 0 || keep_groups < 1 ||
                                         keep_groups > n_groups ||
                                         top > keep_groups * (E / n_groups))))
@@ -228,11 +247,11 @@ extern "C" int zf_moe_route(const void* h, int dtype, const float* router, const
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, 0, stream, (const float*)h, router,
                        bias, ids, weights, T, W, E, top, scoring, correction, n_groups,
-                       keep_groups);
+                       keep_groups, mark_top, normalize, weight_scale, n_extra, extra);
   else
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, router,
                        bias, ids, weights, T, W, E, top, scoring, correction, n_groups,
-                       keep_groups);
+                       keep_groups, mark_top, normalize, weight_scale, n_extra, extra);
   ZF_CHECK_LAUNCH();
 }
 
@@ -303,10 +322,12 @@ __device__ __forceinline__ float row_dot(const T* __restrict__ w, const T* __res
 template <typename T, bool GATED>
 __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_gate_up_kernel(
     const T* __restrict__ h, const T* __restrict__ gate_up, const int* __restrict__ ids,
-    T* __restrict__ y, int W, int ff, int slots, float limit, float alpha, float shift, int act) {
+    T* __restrict__ y, int W, int ff, int slots, float limit, float alpha, float shift, int act,
+    int n_experts) {
   extern __shared__ float xs[];                    // the token's row, [W]
   const int ts = blockIdx.x, t = ts / slots;
   const int e = ids != nullptr ? ids[ts] : 0;
+  if (e >= n_experts) return;                      // an output of the router without an expert
   const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
   const T* row = h + (size_t)t * W;
   for (int i = threadIdx.x; i < W; i += blockDim.x) xs[i] = load_as_float<T>(row + i);
@@ -380,7 +401,8 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_gate_up_kernel(
 // gated != 0: gate_up [E, 2 ff, W]; else [E, ff, W] and the plain activation `act`
 extern "C" int zf_moe_gate_up(const void* h, const void* gate_up, int dtype, const int* ids,
                               void* y, int T, int W, int ff, int slots, float limit, float alpha,
-                              float shift, int gated, int act, hipStream_t stream) {
+                              float shift, int gated, int act, int n_experts,
+                              hipStream_t stream) {
   if (T <= 0) return 0;
   if (W <= 0 || ff <= 0 || slots <= 0 || (size_t)W * sizeof(float) > 64 * 1024 || act < 0 ||
       act > 4)
@@ -391,7 +413,7 @@ extern "C" int zf_moe_gate_up(const void* h, const void* gate_up, int dtype, con
 #define MOE_GU_LAUNCH(TT, G)                                                                      \
   hipLaunchKernelGGL((moe_gate_up_kernel<TT, G>), grid, dim3(MOE_WAVES * ZF_WAVE), smem, stream, \
                      (const TT*)h, (const TT*)gate_up, ids, (TT*)y, W, ff, slots, limit, alpha,  \
-                     shift, act)
+                     shift, act, n_experts)
   if (dtype == ZF_F32) {
     if (gated) MOE_GU_LAUNCH(float, true); else MOE_GU_LAUNCH(float, false);
   } else {
@@ -406,7 +428,7 @@ template <typename T>
 __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_down_kernel(
     const T* __restrict__ y, const T* __restrict__ down, const int* __restrict__ ids,
     const float* __restrict__ weights, float* __restrict__ out, int W, int ff, int slots,
-    int add) {
+    int add, int n_experts, const T* __restrict__ h) {
   const int t = blockIdx.x;
   const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
   const int n0 = (blockIdx.y * MOE_WAVES + wave) * MOE_DOWN_PER_WAVE;
@@ -415,13 +437,19 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_down_kernel(
     if (ff % 8 == 0) {
       // the wave's outputs side by side; a lane adds its pieces over all slots (in slot order)
       // before the lanes are added up, so there is one sum over the wave per output
-      float tot[MOE_DOWN_PER_WAVE];
+      float tot[MOE_DOWN_PER_WAVE], same[MOE_DOWN_PER_WAVE];
 #pragma unroll
-      for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) tot[o] = 0.f;
+      for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) tot[o] = same[o] = 0.f;
       for (int s = 0; s < slots; ++s) {
         const int ts = t * slots + s;
         const int e = ids != nullptr ? ids[ts] : 0;
         const float c = weights != nullptr ? weights[ts] : 1.0f;
+        if (e >= n_experts) {                      // no expert: the token's own row, weighted
+#pragma unroll
+          for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o)
+            same[o] = fmaf(c, load_as_float<T>(h + (size_t)t * W + min(n0 + o, W - 1)), same[o]);
+          continue;
+        }
         const T* yr = y + (size_t)ts * ff;
         const T* wr[MOE_DOWN_PER_WAVE];
 #pragma unroll
@@ -452,7 +480,7 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_down_kernel(
       }
 #pragma unroll
       for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) {
-        const float total = wave_sum(tot[o]);
+        const float total = wave_sum(tot[o]) + same[o];
         if (lane == 0 && n0 + o < W) {
           float* dst = out + (size_t)t * W + n0 + o;
           *dst = add ? *dst + total : total;
@@ -466,6 +494,10 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_down_kernel(
     for (int s = 0; s < slots; ++s) {
       const int ts = t * slots + s;
       const int e = ids != nullptr ? ids[ts] : 0;
+      if (e >= n_experts) {
+        total += (weights != nullptr ? weights[ts] : 1.0f) * load_as_float<T>(h + (size_t)t * W + n);
+        continue;
+      }
       const T* wr = down + ((size_t)e * W + n) * ff;
       const T* yr = y + (size_t)ts * ff;
       const float dot = wave_sum(row_dot<T>(wr, yr, ff, lane));
@@ -480,18 +512,19 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_down_kernel(
 
 extern "C" int zf_moe_down(const void* y, const void* down, int dtype, const int* ids,
                            const float* weights, float* out, int T, int W, int ff, int slots,
-                           int add, hipStream_t stream) {
+                           int add, int n_experts, const void* h, hipStream_t stream) {
   if (T <= 0) return 0;
   if (W <= 0 || ff <= 0 || slots <= 0) return -2;
   const int per_wg = MOE_WAVES * MOE_DOWN_PER_WAVE;
   dim3 grid(T, (W + per_wg - 1) / per_wg);
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(MOE_WAVES * ZF_WAVE), 0, stream,
-                       (const float*)y, (const float*)down, ids, weights, out, W, ff, slots, add);
+                       (const float*)y, (const float*)down, ids, weights, out, W, ff, slots, add,
+                       n_experts, (const float*)h);
   else
     hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(MOE_WAVES * ZF_WAVE), 0, stream,
                        (const bf16_t*)y, (const bf16_t*)down, ids, weights, out, W, ff, slots,
-                       add);
+                       add, n_experts, (const bf16_t*)h);
   ZF_CHECK_LAUNCH();
 }
 
@@ -500,26 +533,32 @@ extern "C" int zf_moe_down(const void* y, const void* down, int dtype, const int
 // made (an expert that every token uses)
 template <typename T>
 __global__ void gated_act_kernel(const T* __restrict__ gu, T* __restrict__ out, int ff, size_t n,
-                                 float limit, float alpha, float shift) {
+                                 float limit, float alpha, float shift,
+                                 const float* __restrict__ row_factor, int factor_stride) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const size_t t = i / ff, j = i % ff;
   const float g = load_as_float<T>(gu + t * 2 * ff + j);
   const float u = load_as_float<T>(gu + t * 2 * ff + ff + j);
-  store_from_float<T>(out + i, gated_unit(g, u, limit, alpha, shift));
+  float r = gated_unit(g, u, limit, alpha, shift);
+  if (row_factor != nullptr) r *= row_factor[t * factor_stride];
+  store_from_float<T>(out + i, r);
 }
 
 extern "C" int zf_gated_act(const void* gu, void* out, int dtype, int T, int ff, float limit,
-                            float alpha, float shift, hipStream_t stream) {
+                            float alpha, float shift, const float* row_factor,
+                            int factor_stride, hipStream_t stream) {
   const size_t n = (size_t)T * ff;
   if (n == 0) return 0;
   const unsigned blocks = (unsigned)((n + 255) / 256);
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(gated_act_kernel<float>, dim3(blocks), dim3(256), 0, stream,
-                       (const float*)gu, (float*)out, ff, n, limit, alpha, shift);
+                       (const float*)gu, (float*)out, ff, n, limit, alpha, shift, row_factor,
+                       factor_stride);
   else
     hipLaunchKernelGGL(gated_act_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
-                       (const bf16_t*)gu, (bf16_t*)out, ff, n, limit, alpha, shift);
+                       (const bf16_t*)gu, (bf16_t*)out, ff, n, limit, alpha, shift, row_factor,
+                       factor_stride);
   ZF_CHECK_LAUNCH();
 }
 
@@ -605,7 +644,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ w, const int* __restrict__ tile_expert,
     const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
     const int* __restrict__ n_tiles, void* __restrict__ out, int N, int K, float limit,
-    float alpha, float shift, int act) {
+    float alpha, float shift, int act, int n_experts) {
   constexpr bool GATED = MODE == 1;
   constexpr bool GATHER = MODE != 0;            // rows of h found through the sort
   __shared__ __attribute__((aligned(16))) bf16_t as[MOE_TILE_ROWS * MOE_LD];
@@ -615,6 +654,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   const int tile = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
   if (tile >= n_tiles[0]) return;
   const int e = tile_expert[tile], row0 = tile_row0[tile], nrows = tile_rows[tile];
+  if (e >= n_experts) return;                      // an output of the router without an expert
   const int c0 = blockIdx.y * 64 * (GATED ? MOE_HALF : MOE_NB);
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wm = wave / 2, wn = wave % 2;
@@ -729,7 +769,7 @@ extern "C" int zf_moe_grouped(const void* a, long long lda, const int* sorted, i
                               const void* w, const int* tile_expert, const int* tile_row0,
                               const int* tile_rows, const int* n_tiles, void* out, int max_tiles,
                               int N, int K, int mode, float limit, float alpha, float shift,
-                              int act, hipStream_t stream) {
+                              int act, int n_experts, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (N <= 0 || K <= 0 || K % 8 != 0 || top <= 0 || mode < 0 || mode > 2 || act < 0 || act > 4)
     return -2;
@@ -738,7 +778,7 @@ extern "C" int zf_moe_grouped(const void* a, long long lda, const int* sorted, i
   hipLaunchKernelGGL(moe_grouped_kernel<MODE>, dim3(max_tiles, (N + (COLS) - 1) / (COLS)),       \
                      dim3(256), 0, stream, (const bf16_t*)a, lda, sorted, top, (const bf16_t*)w, \
                      tile_expert, tile_row0, tile_rows, n_tiles, out, N, K, limit, alpha, shift, \
-                     act)
+                     act, n_experts)
   if (mode == 1) MOE_GROUPED_LAUNCH(1, 64 * MOE_HALF);
   else if (mode == 2) MOE_GROUPED_LAUNCH(2, 64 * MOE_NB);
   else MOE_GROUPED_LAUNCH(0, 64 * MOE_NB);
@@ -747,13 +787,17 @@ extern "C" int zf_moe_grouped(const void* a, long long lda, const int* sorted, i
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const float* __restrict__ o, const int* __restrict__ place, const float* __restrict__ weights,
-    float* __restrict__ out, int W, int slots, int add) {
+    float* __restrict__ out, int W, int slots, int add, const int* __restrict__ ids,
+    int n_experts, const bf16_t* __restrict__ h) {
   const int t = blockIdx.x;
   for (int n = blockIdx.y * blockDim.x + threadIdx.x; n < W; n += gridDim.y * blockDim.x) {
     float total = 0.f;
     for (int s = 0; s < slots; ++s) {
       const int ts = t * slots + s;
-      total += weights[ts] * o[(size_t)place[ts] * W + n];
+      // an output of the router without an expert hands the token's own row on
+      const float v = (ids != nullptr && ids[ts] >= n_experts)
+          ? bf16_to_float(h[(size_t)t * W + n]) : o[(size_t)place[ts] * W + n];
+      total += weights[ts] * v;
     }
     float* dst = out + (size_t)t * W + n;
     *dst = add ? *dst + total : total;
@@ -761,12 +805,13 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
 }
 
 extern "C" int zf_moe_combine(const float* o, const int* place, const float* weights, float* out,
-                              int T, int W, int slots, int add, hipStream_t stream) {
+                              int T, int W, int slots, int add, const int* ids, int n_experts,
+                              const void* h, hipStream_t stream) {
   if (T <= 0) return 0;
   if (W <= 0 || slots <= 0) return -2;
   int gy = (W + 255) / 256;
   if (gy > 64) gy = 64;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(T, gy), dim3(256), 0, stream, o, place, weights,
-                     out, W, slots, add);
+                     out, W, slots, add, ids, n_experts, (const bf16_t*)h);
   ZF_CHECK_LAUNCH();
 }

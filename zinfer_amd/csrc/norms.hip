@@ -322,3 +322,96 @@ extern "C" int zf_embed_position(const void* table, const void* pos_table, int t
                        scale);
   ZF_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------- several copies of the residual stream
+// The stream is kept in S copies x_1 .. x_S, [S, T, W] floats.  Around a sublayer, row by row
+// (a workgroup a row, a thread the same columns of all copies, everything 32-bit):
+//
+//   write:  x_t <- sum_s M[s, t] x_s + b[t] y   for all t from the old copies,
+//           y = c0 y0 (+ c1 y1): the sublayer's output, in one branch or two
+//   read:   u = sum_s a[s] x_s (the new copies), then out = u / sqrt(mean(u^2) + eps) * gain in
+//           the products' type, or (no gain) out = u as floats
+//
+// Either half may be left out: the read alone before a layer's first sublayer and for the sum
+// of the copies at the end, both between two sublayers.  The sums run over s in ascending order.
+#define STREAMS_MAX 8
+
+template <typename TO>
+__global__ __launch_bounds__(256) void streams_step_kernel(
+    float* __restrict__ x, long long copy_stride, int S, const float* __restrict__ y0,
+    const float* __restrict__ y1, float c0, float c1, const float* __restrict__ M,
+    const float* __restrict__ b, const float* __restrict__ a, const float* __restrict__ gain,
+    float eps, TO* __restrict__ out, int W, int do_read) {
+#pragma clang fp contract(off)
+  extern __shared__ float u_row[];
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v[STREAMS_MAX];
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s) v[s] = s < S ? x[s * copy_stride + row + i] : 0.f;
+    if (y0 != nullptr) {
+      float y = c0 * y0[row + i];
+      if (y1 != nullptr) y = y + c1 * y1[row + i];
+      float n[STREAMS_MAX];
+#pragma unroll
+      for (int t = 0; t < STREAMS_MAX; ++t) {
+        if (t >= S) continue;
+        float acc = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; ++s)
+          if (s < S) acc = acc + M[s * S + t] * v[s];
+        n[t] = acc + b[t] * y;
+      }
+#pragma unroll
+      for (int t = 0; t < STREAMS_MAX; ++t)
+        if (t < S) {
+          v[t] = n[t];
+          x[t * copy_stride + row + i] = n[t];
+        }
+    }
+    if (do_read) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < STREAMS_MAX; ++s)
+        if (s < S) u = u + (a != nullptr ? a[s] : 1.0f) * v[s];
+      if (gain == nullptr) {
+        store_from_float<TO>(out + row + i, u);
+      } else {
+        u_row[i] = u;
+        ss += u * u;
+      }
+    }
+  }
+  if (!do_read || gain == nullptr) return;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  // (a thread reads back the columns it wrote itself)
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    store_from_float<TO>(out + row + i, u_row[i] * inv * gain[i]);
+}
+
+// x [S, T, W] (copy_stride elements from one copy to the next).  y0 null: no write; else y1
+// may be null.  do_read 0: no read; else `a` may be null (all ones) and `gain` may be null
+// (out float32 = u; out_dtype must then be float32).
+extern "C" int zf_streams_step(float* x, long long copy_stride, int S, const float* y0,
+                               const float* y1, float c0, float c1, const float* M,
+                               const float* b, const float* a, const float* gain, float eps,
+                               void* out, int out_dtype, int T, int W, int do_read,
+                               hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (S < 1 || S > STREAMS_MAX || W <= 0 || W > 16384 || (y0 == nullptr && !do_read) ||
+      (y0 != nullptr && (M == nullptr || b == nullptr)) || (do_read && out == nullptr) ||
+      (do_read && gain == nullptr && out_dtype != ZF_F32))
+    return -2;
+  const size_t smem = (size_t)W * sizeof(float);
+  if (out_dtype == ZF_F32)
+    hipLaunchKernelGGL(streams_step_kernel<float>, dim3(T), dim3(256), smem, stream, x,
+                       copy_stride, S, y0, y1, c0, c1, M, b, a, gain, eps, (float*)out, W, do_read);
+  else
+    hipLaunchKernelGGL(streams_step_kernel<bf16_t>, dim3(T), dim3(256), smem, stream, x,
+                       copy_stride, S, y0, y1, c0, c1, M, b, a, gain, eps, (bf16_t*)out, W,
+                       do_read);
+  ZF_CHECK_LAUNCH();
+}

@@ -149,9 +149,12 @@ class Engine:
                 if e.layer == layer and e.cache_of is None]
         if not runs:
             raise StepError(f"no run of the schedule has layer {layer} with a cache of its own")
-        T, width = hidden.shape
-        if width != spec.hidden_size or T < 1:
-            raise StepError(f"hidden is {tuple(hidden.shape)}, the stream is [T, {spec.hidden_size}]")
+        # (a model whose stream lies in several copies takes and returns [copies, T, hidden])
+        lead = (spec.streams,) if spec.streams is not None else ()
+        T, width = hidden.shape[-2:] if hidden.dim() >= 2 else (0, 0)
+        if width != spec.hidden_size or T < 1 or tuple(hidden.shape[:-2]) != lead:
+            raise StepError(f"hidden is {tuple(hidden.shape)}, the stream is "
+                            f"{list(lead) + ['T', spec.hidden_size]}")
         rid = object()
         entry = StepEntry(rid, [0] * T, [])
         self._check_entries([entry])
@@ -160,7 +163,7 @@ class Engine:
         self._reserve([(rid, T)])
         try:
             ctx = self._build_context([entry])
-            x = ctx.scratch("residual", (T, spec.hidden_size), torch.float32)
+            x = ctx.scratch("residual", lead + (T, spec.hidden_size), torch.float32)
             x.copy_(hidden)
             ctx.norm_ready = ctx.norm_after_block = None
             self.model.blocks[layer].forward(x, ctx, self.views[runs[0]])

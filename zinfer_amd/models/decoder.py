@@ -19,19 +19,28 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec, ctx: BuildContext):
         self.spec = spec
         self.ctx = ctx
-        self.blocks = [build_part("block", b, ctx, spec.layer_prefix.format(i))
-                       for i, b in enumerate(spec.layers)]
+        numbers = spec.layer_numbers if spec.layer_numbers is not None \
+            else tuple(range(len(spec.layers)))
+        if len(numbers) != len(spec.layers):
+            raise ConfigError(f"{len(spec.layers)} layers go by {len(numbers)} numbers")
+        self.blocks = [build_part("block", b, ctx, spec.layer_prefix.format(n))
+                       for n, b in zip(numbers, spec.layers)]
         self.final_norm = build_part("norm", spec.final_norm, ctx, spec.final_norm_prefix)
         self.graph_safe = self.final_norm.graph_safe and all(b.graph_safe for b in self.blocks)
         # (inspection) called with (schedule position, the stream) behind every run of a block
         self.layer_probe = None
         # embedding, row gather and head are the model's own launches
         self.kernel_modules = tuple(sorted(
-            {"elementwise", "gemm"} | ({"norms"} if spec.position_table_name is not None else set())
+            {"elementwise", "gemm"}
+            | ({"norms"} if spec.position_table_name is not None or spec.streams is not None
+               else set())
             | set(self.final_norm.kernel_modules)
             | {m for b in self.blocks for m in b.kernel_modules}))
         if spec.position_table_name is not None and spec.sinusoidal_positions is not None:
             raise ConfigError("a learned position table or computed position vectors, not both")
+        if spec.streams is not None and (spec.streams < 1 or spec.reentry_name is not None):
+            raise ConfigError("a stream in several copies needs at least one copy, and no run "
+                              "re-enters the embedding's output")
         if any(e.reentry for e in spec.schedule) and spec.reentry_name is None:
             raise ConfigError("a run of the schedule re-enters the embedding's output, but the "
                               "model names no matrix for it")
@@ -113,13 +122,25 @@ class DecoderModel:
         return [None if e.cache_of is not None else self.blocks[e.layer].cache_need()
                 for e in self.spec.schedule]
 
+    def _sum(self, copies: torch.Tensor, step) -> torch.Tensor:
+        """The copies of the stream added up, [T, hidden] float32."""
+        total = step.scratch("residual_sum", tuple(copies.shape[1:]), torch.float32)
+        ops.streams_step(copies, read=True, out=total)
+        return total
+
     # ---------------------------------------------------------------- forward
     def forward(self, step, caches) -> torch.Tensor:
         """Runs the tokens of ``step`` and returns float32 logits [len(step.want_rows), V].
         ``caches[pos]`` is the cache view of schedule position ``pos`` (or None)."""
         s = self.spec
         T = step.n_tokens
-        x = step.scratch("residual", (T, s.hidden_size), torch.float32)
+        copies = None
+        if s.streams is not None:
+            # the stream in several copies, all equal to the embedding's output at the start
+            copies = step.scratch("residual", (s.streams, T, s.hidden_size), torch.float32)
+            x = copies[0]
+        else:
+            x = step.scratch("residual", (T, s.hidden_size), torch.float32)
         if self.position_table is not None:
             ops.embed_position(self.embedding, step.token_ids, self.position_table,
                                step.positions, x, float(s.embedding_multiplier))
@@ -133,6 +154,10 @@ class DecoderModel:
             # the stream as the embedding left it, for the runs that re-enter it
             x0 = step.scratch("embedding_out", (T, s.hidden_size), torch.float32)
             x0.copy_(x)
+        if copies is not None:
+            for c in range(1, s.streams):
+                copies[c].copy_(x)
+            x = copies
         step.norm_ready = None
         for pos, e in enumerate(s.schedule):
             if e.reentry:
@@ -153,8 +178,10 @@ class DecoderModel:
             step.norm_after_block = after
             self.blocks[e.layer].forward(x, step, caches[pos])
             if self.layer_probe is not None:
-                self.layer_probe(pos, x)
+                self.layer_probe(pos, x if copies is None else self._sum(copies, step))
         left, step.norm_ready, step.norm_after_block = step.norm_ready, None, None
+        if copies is not None:
+            x, left = self._sum(copies, step), None
         n_rows = step.n_want
         logits = step.scratch("logits", (n_rows, s.vocab_size), torch.float32)
         if n_rows == 0:

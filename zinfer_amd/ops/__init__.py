@@ -1726,14 +1726,16 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
 MOE_MAX_EXPERTS = 1024
 
 
-ROUTER_SCORINGS = {"softmax": 0, "sigmoid": 1}
+ROUTER_SCORINGS = {"softmax": 0, "sigmoid": 1, "softmax_all": 2}
 
 
 @_launches("other")
 def moe_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor],
               ids: torch.Tensor, weights: torch.Tensor, scoring: str = "softmax",
               correction: Optional[torch.Tensor] = None,
-              groups: Optional[Tuple[int, int]] = None) -> None:
+              groups: Optional[Tuple[int, int]] = None, group_mark: int = 2,
+              normalize: bool = True, weight_scale: float = 1.0,
+              extra: Optional[torch.Tensor] = None) -> None:
     """Per row of ``h`` [T, W]: z = router h + bias in 32-bit (router float32 [E, W]); ``ids``
     [T, top] int32 receives the ``top`` chosen experts (the lower index wins a tie).
     ``scoring`` "softmax": the largest z are chosen and ``weights`` [T, top] float32 is the
@@ -1741,16 +1743,30 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     (float32 [E], or none); with ``groups`` = (count, keep) the experts form ``count`` equal
     groups of neighbours, a group is marked by its two largest choice scores added, and only
     experts of the ``keep`` best groups can be chosen; the weights are the chosen s over their
-    sum (+ 1e-20)."""
-    _need_gpu(h, router, bias, ids, weights, correction)
+    sum (+ 1e-20).  "softmax_all": the same with s = softmax(z) over all E outputs.
+    ``group_mark`` 1: a group is marked by its largest choice score alone.  ``normalize`` False:
+    the weights are the chosen s themselves; either way times ``weight_scale``.  ``extra``
+    float32 [T, n]: the router has n more rows behind its E outputs, which are no experts; the
+    sigmoids of their products with h go there (a gate a token that rides with the router)."""
+    _need_gpu(h, router, bias, ids, weights, correction, extra)
     _i32(ids, "ids")
     T, W = h.shape
-    E = router.shape[0]
+    n_extra = 0
+    if extra is not None:
+        if extra.dim() != 2 or extra.shape[0] != T or extra.dtype != torch.float32 \
+                or not extra.is_contiguous() or extra.shape[1] >= router.shape[0]:
+            raise KernelUnavailable(f"moe_route: extra {tuple(extra.shape)} {extra.dtype} must be "
+                                    "float32 [T, n], n rows of the router behind the experts'")
+        n_extra = extra.shape[1]
+    E = router.shape[0] - n_extra
     top = ids.shape[1] if ids.dim() == 2 else 0
     count, keep = groups if groups is not None else (0, 0)
-    if router.dtype != torch.float32 or router.shape != (E, W) or ids.shape != (T, top) \
+    if router.dtype != torch.float32 or router.shape != (E + n_extra, W) \
+            or not router.is_contiguous() or ids.shape != (T, top) \
             or weights.shape != (T, top) or weights.dtype != torch.float32 \
-            or not 0 < top <= E <= MOE_MAX_EXPERTS or scoring not in ROUTER_SCORINGS \
+            or not 0 < top <= E or E + n_extra > MOE_MAX_EXPERTS \
+            or scoring not in ROUTER_SCORINGS or group_mark not in (1, 2) \
+            or (scoring == "softmax" and (not normalize or n_extra)) \
             or (bias is not None and (bias.dtype != torch.float32 or bias.shape != (E,))) \
             or (correction is not None and (correction.dtype != torch.float32
                                             or correction.shape != (E,))) \
@@ -1763,18 +1779,21 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     lib = build.load("moe")
     _check(lib.zf_moe_route(_ptr(h), _dt(h), _ptr(router), _ptr(bias), _ptr(ids), _ptr(weights),
                             T, W, E, top, ROUTER_SCORINGS[scoring], _ptr(correction), int(count),
-                            int(keep), _stream()), "moe_route")
+                            int(keep), int(group_mark), 1 if normalize else 0,
+                            ctypes.c_float(weight_scale), n_extra, _ptr(extra), _stream()),
+           "moe_route")
 
 
 @_launches("products")
 def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, ids: Optional[torch.Tensor],
                 y: torch.Tensor, limit: float, alpha: float, shift: float,
-                act: Optional[str] = None) -> None:
+                act: Optional[str] = None, n_identity: int = 0) -> None:
     """y[t, s, :] = act(expert ids[t, s] of ``gate_up`` [E, 2 ff, W] applied to h[t]) with
     g = min(gate, limit), u = clamp(up, -limit, limit) (no clamp if limit <= 0) and
     act = g * sigmoid(alpha g) * (u + shift).  With ``act`` (one of ``ACTIVATIONS``) the experts
     have no gate: ``gate_up`` is [E, ff, W] and y = act(up h).  ``ids`` None: expert 0 for every
-    token."""
+    token.  ``n_identity``: ids from E up to E + n_identity - 1 name no expert; their rows of y
+    are left alone."""
     _need_gpu(h, gate_up, ids, y)
     T, W = h.shape
     if y.dim() != 3 or gate_up.dim() != 3:
@@ -1794,17 +1813,20 @@ def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, ids: Optional[torch.Tens
     _check(lib.zf_moe_gate_up(_ptr(h), _ptr(gate_up), _dt(h), _ptr(ids), _ptr(y), T, W, ff,
                               slots, ctypes.c_float(limit), ctypes.c_float(alpha),
                               ctypes.c_float(shift), 0 if act is not None else 1,
-                              ACTIVATIONS[act] if act is not None else 0, _stream()),
+                              ACTIVATIONS[act] if act is not None else 0,
+                              gate_up.shape[0] if n_identity else (1 << 30), _stream()),
            "moe_gate_up")
 
 
 @_launches("products")
 def moe_down(y: torch.Tensor, down: torch.Tensor, ids: Optional[torch.Tensor],
-             weights: Optional[torch.Tensor], out: torch.Tensor, add: bool = False) -> None:
+             weights: Optional[torch.Tensor], out: torch.Tensor, add: bool = False,
+             identity: Optional[torch.Tensor] = None) -> None:
     """out[t] (=, or with ``add`` +=) sum over s of weights[t, s] * down[ids[t, s]] y[t, s], in
     slot order and 32-bit; ``down`` [E, W, ff], ``out`` float32 [T, W].  ``ids`` None: expert
-    0; ``weights`` None: 1."""
-    _need_gpu(y, down, ids, weights, out)
+    0; ``weights`` None: 1.  ``identity`` [T, W] (the experts' input): an id from E on names no
+    expert, and its term is weights[t, s] * identity[t]."""
+    _need_gpu(y, down, ids, weights, out, identity)
     if y.dim() != 3 or down.dim() != 3:
         raise KernelUnavailable("moe_down: y [T, slots, ff], down [E, W, ff]")
     T, slots, ff = y.shape
@@ -1815,26 +1837,35 @@ def moe_down(y: torch.Tensor, down: torch.Tensor, ids: Optional[torch.Tensor],
             or out.dtype != torch.float32 or (ids is not None and ids.shape != (T, slots)) \
             or (ids is None and down.shape[0] != 1) \
             or (weights is not None and (weights.shape != (T, slots)
-                                         or weights.dtype != torch.float32)):
+                                         or weights.dtype != torch.float32)) \
+            or (identity is not None and (identity.shape != (T, W) or identity.dtype != y.dtype
+                                          or not identity.is_contiguous())):
         raise KernelUnavailable(f"moe_down: y {tuple(y.shape)} {y.dtype}, down "
                                 f"{tuple(down.shape)} {down.dtype}, out {tuple(out.shape)}")
     lib = build.load("moe")
     _check(lib.zf_moe_down(_ptr(y), _ptr(down), _dt(y), _ptr(ids), _ptr(weights), _ptr(out), T,
-                           W, ff, slots, 1 if add else 0, _stream()), "moe_down")
+                           W, ff, slots, 1 if add else 0,
+                           down.shape[0] if identity is not None else (1 << 30), _ptr(identity),
+                           _stream()), "moe_down")
 
 
 @_launches("norm_rope_write")
 def gated_act(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float,
-              shift: float) -> None:
+              shift: float, row_factor: Optional[torch.Tensor] = None) -> None:
     """out[t, j] = g * sigmoid(alpha g) * (u + shift) with g = min(gate_up[t, j], limit) and
-    u = clamp(gate_up[t, ff + j], -limit, limit) (no clamp if limit <= 0)."""
-    _need_gpu(gate_up, out)
+    u = clamp(gate_up[t, ff + j], -limit, limit) (no clamp if limit <= 0); times
+    ``row_factor[t]`` (float32 [T] or a column of a float32 matrix) if given."""
+    _need_gpu(gate_up, out, row_factor)
     T, ff = out.shape
-    if gate_up.shape != (T, 2 * ff) or gate_up.dtype != out.dtype:
+    if gate_up.shape != (T, 2 * ff) or gate_up.dtype != out.dtype \
+            or (row_factor is not None and (row_factor.dtype != torch.float32
+                                            or row_factor.dim() != 1 or row_factor.shape[0] != T)):
         raise KernelUnavailable(f"gated_act: gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)}")
     lib = build.load("moe")
     _check(lib.zf_gated_act(_ptr(gate_up), _ptr(out), _dt(out), T, ff, ctypes.c_float(limit),
-                            ctypes.c_float(alpha), ctypes.c_float(shift), _stream()), "gated_act")
+                            ctypes.c_float(alpha), ctypes.c_float(shift), _ptr(row_factor),
+                            int(row_factor.stride(0)) if row_factor is not None else 0,
+                            _stream()), "gated_act")
 
 
 MOE_TILE_ROWS = 128           # MOE_TILE_ROWS in moe.hip
@@ -1852,24 +1883,27 @@ def moe_grouped_covers(h: torch.Tensor, gate_up: torch.Tensor, act: Optional[str
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
                 weights: torch.Tensor, y: torch.Tensor, out: torch.Tensor, limit: float,
                 alpha: float, shift: float, add: bool = False,
-                act: Optional[str] = None) -> None:
+                act: Optional[str] = None, n_identity: int = 0) -> None:
     """out[t] (=, +=) sum over s of weights[t, s] * expert ids[t, s] applied to h[t]
     (``moe_gate_up`` then ``moe_down``), with ``y`` [T, top, ff] as work space.  A few tokens
     stream each chosen expert's matrices (one workgroup row per token and slot); more tokens,
     in bfloat16, are sorted by expert and run through MFMA tiles of ``MOE_TILE_ROWS`` pairs
     (``moe_sort``, ``moe_grouped`` twice, ``moe_combine``).  Either way a token's result
-    depends on that token alone.  ``act``: experts without a gate (see ``moe_gate_up``)."""
+    depends on that token alone.  ``act``: experts without a gate (see ``moe_gate_up``).
+    ``n_identity``: ids from E up to E + n_identity - 1 name no expert; such a term of the sum is
+    the weight times h[t] itself."""
     T, W = h.shape
     if T > MOE_STREAM_MAX_TOKENS and moe_grouped_covers(h, gate_up, act):
-        moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add, act)
+        moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add, act,
+                    n_identity)
         return
-    moe_gate_up(h, gate_up, ids, y, limit, alpha, shift, act)
-    moe_down(y, down, ids, weights, out, add=add)
+    moe_gate_up(h, gate_up, ids, y, limit, alpha, shift, act, n_identity)
+    moe_down(y, down, ids, weights, out, add=add, identity=h if n_identity else None)
 
 
 @_launches("products")
 def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add=False,
-                act: Optional[str] = None) -> None:
+                act: Optional[str] = None, n_identity: int = 0) -> None:
     """The many-token form of ``moe_experts`` (bfloat16; see there)."""
     _need_gpu(h, gate_up, down, ids, weights, y, out)
     _i32(ids, "ids")
@@ -1883,13 +1917,15 @@ def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add
             or ids.shape != (T, top) or weights.shape != (T, top) \
             or weights.dtype != torch.float32 or y.dtype != torch.bfloat16 \
             or y.numel() != T * top * ff or not y.is_contiguous() \
-            or out.shape != (T, W) or out.dtype != torch.float32 or not 0 < E <= MOE_MAX_EXPERTS \
+            or out.shape != (T, W) or out.dtype != torch.float32 \
+            or not 0 < E <= E + n_identity <= MOE_MAX_EXPERTS or not h.is_contiguous() \
             or (act is not None and act not in ACTIVATIONS):
         raise KernelUnavailable(f"moe_grouped: h {tuple(h.shape)} {h.dtype}, gate_up "
                                 f"{tuple(gate_up.shape)}, down {tuple(down.shape)}, ids "
                                 f"{tuple(ids.shape)}, y {tuple(y.shape)} {y.dtype}")
     P = T * top
-    max_tiles = (P + MOE_TILE_ROWS - 1) // MOE_TILE_ROWS + E
+    EA = E + n_identity           # the sort's buckets: the ids that name no expert have theirs
+    max_tiles = (P + MOE_TILE_ROWS - 1) // MOE_TILE_ROWS + EA
     # places of the pairs, the tiles' list and the experts' 32-bit outputs, kept across steps
     table = _workspace("moe_table", 2 * P + 3 * max_tiles + 4, torch.int32, h.device)
     o = _workspace("moe_out", P * W, torch.float32, h.device)
@@ -1900,20 +1936,21 @@ def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add
     n_tiles = table[t0 + 3 * max_tiles:]
     lib = build.load("moe")
     st = _stream()
-    _check(lib.zf_moe_sort(_ptr(ids), P, E, _ptr(sorted_), _ptr(place), _ptr(tile_expert),
+    _check(lib.zf_moe_sort(_ptr(ids), P, EA, _ptr(sorted_), _ptr(place), _ptr(tile_expert),
                            _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles), st), "moe_sort")
     lim, al, sh = ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift)
     kind = ACTIVATIONS[act] if act is not None else 0
     _check(lib.zf_moe_grouped(_ptr(h), ctypes.c_longlong(W), _ptr(sorted_), top, _ptr(gate_up),
                               _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles),
                               _ptr(y), max_tiles, ff, W, 2 if act is not None else 1, lim, al, sh,
-                              kind, st), "moe_grouped (gate, up)")
+                              kind, E, st), "moe_grouped (gate, up)")
     _check(lib.zf_moe_grouped(_ptr(y), ctypes.c_longlong(ff), _ptr(sorted_), top, _ptr(down),
                               _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles),
-                              _ptr(o), max_tiles, W, ff, 0, lim, al, sh, 0, st),
+                              _ptr(o), max_tiles, W, ff, 0, lim, al, sh, 0, E, st),
            "moe_grouped (down)")
     _check(lib.zf_moe_combine(_ptr(o), _ptr(place), _ptr(weights), _ptr(out), T, W, top,
-                              1 if add else 0, st), "moe_combine")
+                              1 if add else 0, _ptr(ids) if n_identity else None, E,
+                              _ptr(h) if n_identity else None, st), "moe_combine")
 
 
 # ------------------------------------------------------------------------- sampling
@@ -2003,12 +2040,16 @@ class RowSegment:
     elements of a head below ``skip`` are not written.  The rest goes to ``dst``: plain rows
     [T, ...] where head h starts at column dst_off + h * dst_hd (dst_hd None: hd - skip), or
     (``pool_heads`` given) a pool of blocks [page, kv head] of rows of dst_hd elements (laid out as
-    ``masked_pool_from_rows`` says) at the token's slot, from column dst_off of the row on."""
+    ``masked_pool_from_rows`` says) at the token's slot, from column dst_off of the row on.
+    ``bias`` [width] float32 is added to the source's values before anything else.  ``per_head``:
+    the norm runs over every head on its own and ``gain`` is [hd], one for all heads.
+    ``interleaved``: the rotated pairs are the neighbours (2i, 2i + 1), pair i by freq[i]."""
 
     def __init__(self, src_off: int, width: int, dst: torch.Tensor, *, gain=None, eps: float = 0.0,
                  hd: Optional[int] = None, rot_off: int = 0, rot_dims: int = 0, freq=None,
                  mag: float = 1.0, skip: int = 0, dst_off: int = 0, dst_hd: Optional[int] = None,
-                 pool_heads: Optional[int] = None):
+                 pool_heads: Optional[int] = None, bias=None, per_head: bool = False,
+                 interleaved: bool = False):
         self.src_off, self.width, self.dst = int(src_off), int(width), dst
         self.gain, self.eps = gain, float(eps)
         self.hd = int(hd) if hd is not None else int(width)
@@ -2016,6 +2057,7 @@ class RowSegment:
         self.skip, self.dst_off = int(skip), int(dst_off)
         self.dst_hd = int(dst_hd) if dst_hd is not None else self.hd - self.skip
         self.pool_heads = pool_heads
+        self.bias, self.per_head, self.interleaved = bias, bool(per_head), bool(interleaved)
 
 
 PROJECT_ROWS_MAX_SEGMENTS = 4
@@ -2045,7 +2087,10 @@ def project_rows(src: torch.Tensor, positions: torch.Tensor, slot_mapping: Optio
             and g.rot_off + g.rot_dims <= g.hd and 0 <= g.skip < g.hd \
             and g.dst.is_cuda and g.dst.dtype == src.dtype and g.dst_off >= 0 \
             and (g.gain is None or (g.gain.is_cuda and g.gain.dtype == torch.float32
-                                    and g.gain.shape == (g.width,) and g.gain.is_contiguous())) \
+                                    and g.gain.shape == ((g.hd if g.per_head else g.width),)
+                                    and g.gain.is_contiguous())) \
+            and (g.bias is None or (g.bias.is_cuda and g.bias.dtype == torch.float32
+                                    and g.bias.shape == (g.width,) and g.bias.is_contiguous())) \
             and (g.rot_dims == 0 or (g.freq is not None and g.freq.is_cuda
                                      and g.freq.dtype == torch.float32
                                      and g.freq.shape == (g.rot_dims // 2,)))
@@ -2066,10 +2111,12 @@ def project_rows(src: torch.Tensor, positions: torch.Tensor, slot_mapping: Optio
                                     f"source {tuple(src.shape)} or destination "
                                     f"{tuple(g.dst.shape)} {g.dst.dtype}")
         ints += [g.src_off, g.width, g.hd, g.rot_off, g.rot_dims, g.skip, 1 if pool else 0,
-                 g.dst_off, g.dst_hd, g.pool_heads or 0, 0]
+                 g.dst_off, g.dst_hd, g.pool_heads or 0,
+                 (1 if g.per_head else 0) | (2 if g.interleaved else 0)]
         floats += [g.eps, g.mag]
         ptrs += [g.gain.data_ptr() if g.gain is not None else None,
-                 g.freq.data_ptr() if g.rot_dims else None, g.dst.data_ptr()]
+                 g.freq.data_ptr() if g.rot_dims else None, g.dst.data_ptr(),
+                 g.bias.data_ptr() if g.bias is not None else None]
     lib = build.load("masked_attention")
     _check(lib.zf_project_rows(
         _ptr(src), _dt(src), ctypes.c_longlong(stride), _ptr(positions), _ptr(slot_mapping), T,
@@ -2510,3 +2557,185 @@ def head_norm_gate(o: torch.Tensor, gain: torch.Tensor, gate: torch.Tensor, out:
                                  ctypes.c_longlong(_columns(gate, "head_norm_gate: gate")),
                                  _ptr(out), _dt(out), T, H, dv, ctypes.c_float(eps), _stream()),
            "head_norm_gate")
+
+
+# ------------------------------------------------------------------------- the residual stream in several copies
+STREAMS_MAX = 8               # STREAMS_MAX in norms.hip
+STREAMS_MAX_WIDTH = 16384
+
+
+@_launches("norm_rope_write")
+def streams_step(x: torch.Tensor, branches=(), mix: Optional[torch.Tensor] = None,
+                 out_coef: Optional[torch.Tensor] = None, *, read: bool = False,
+                 in_coef: Optional[torch.Tensor] = None, gain: Optional[torch.Tensor] = None,
+                 eps: float = 0.0, out: Optional[torch.Tensor] = None) -> None:
+    """Around a sublayer of a model whose residual stream is kept in S copies ``x`` float32
+    [S, T, W] (a view whose copies are contiguous [T, W] matrices a fixed distance apart), row by
+    row, all 32-bit.  With ``branches`` = one or two (y float32 [T, W], factor): y = the sum of
+    factor * y, and x_t <- sum_s mix[s, t] x_s + out_coef[t] * y for all t at once from the old
+    copies (``mix`` float32 [S, S], ``out_coef`` float32 [S]).  With ``read``: u = sum_s
+    in_coef[s] x_s over the (new) copies (``in_coef`` None: all ones), and ``out`` [T, W] =
+    u / sqrt(mean(u^2) + eps) * gain in out's type, or (``gain`` None) u itself as float32.
+    Both halves in one launch when both are asked for."""
+    _need_gpu(x, mix, out_coef, in_coef, gain, out, *[y for y, _ in branches])
+    if x.dim() != 3 or x.dtype != torch.float32 or x.stride(2) != 1 or x.stride(1) != x.shape[2]:
+        raise KernelUnavailable(f"streams_step: x {tuple(x.shape)} {x.dtype} must be float32 "
+                                "[S, T, W] with contiguous copies")
+    S, T, W = x.shape
+    ok = 1 <= S <= STREAMS_MAX and 0 < W <= STREAMS_MAX_WIDTH and len(branches) <= 2 \
+        and (branches or read)
+    for y, _ in branches:
+        ok = ok and y.shape == (T, W) and y.dtype == torch.float32 and y.is_contiguous()
+    if branches:
+        ok = ok and mix is not None and out_coef is not None and mix.shape == (S, S) \
+            and out_coef.shape == (S,) and mix.dtype == torch.float32 \
+            and out_coef.dtype == torch.float32 and mix.is_contiguous()
+    if read:
+        ok = ok and out is not None and out.shape == (T, W) and out.is_contiguous() \
+            and (in_coef is None or (in_coef.shape == (S,) and in_coef.dtype == torch.float32)) \
+            and (gain is None or (gain.shape == (W,) and gain.dtype == torch.float32)) \
+            and (gain is not None or out.dtype == torch.float32)
+    if not ok:
+        raise KernelUnavailable(f"streams_step: x {tuple(x.shape)}, {len(branches)} branches, "
+                                f"read {read}: up to {STREAMS_MAX} copies of up to "
+                                f"{STREAMS_MAX_WIDTH} columns, float32 coefficients [S], [S, S]")
+    y0 = branches[0][0] if branches else None
+    y1 = branches[1][0] if len(branches) > 1 else None
+    c0 = float(branches[0][1]) if branches else 0.0
+    c1 = float(branches[1][1]) if len(branches) > 1 else 0.0
+    lib = build.load("norms")
+    _check(lib.zf_streams_step(_ptr(x), ctypes.c_longlong(x.stride(0) if S > 1 else T * W), S,
+                               _ptr(y0), _ptr(y1), ctypes.c_float(c0), ctypes.c_float(c1),
+                               _ptr(mix), _ptr(out_coef), _ptr(in_coef), _ptr(gain),
+                               ctypes.c_float(eps), _ptr(out), _dt(out) if out is not None else 0,
+                               T, W, 1 if read else 0, _stream()), "streams_step")
+
+
+# ------------------------------------------------------------------------- the gated delta rule
+DELTA_MAX_KEY_DIM = 256
+DELTA_CHANNELS = (8, 12, 16)      # key channels a thread holds (instantiations in delta.hip)
+DELTA_MAX_LANES = 16              # lanes that share a column's key channels
+
+
+def delta_plan(key_dim: int) -> Tuple[int, int]:
+    """(channels a thread, lanes a column) for heads of ``key_dim``: the padded key size
+    channels * lanes is the smallest of 8, 12, 16, 24, 32, 48, ... that holds the head, and as
+    many lanes (a power of two, at most ``DELTA_MAX_LANES``) share a column as leave a thread
+    at least 8 channels.  A function of the key size alone: a request's state is laid out by it."""
+    best = None
+    for r in DELTA_CHANNELS:
+        lanes = 1
+        while lanes <= DELTA_MAX_LANES:
+            if r * lanes >= key_dim:
+                if best is None or (r * lanes, -lanes) < (best[0] * best[1], -best[1]):
+                    best = (r, lanes)
+                break
+            lanes *= 2
+    if best is None:
+        raise KernelUnavailable(f"delta rule: key size {key_dim} beyond {DELTA_MAX_KEY_DIM}")
+    return best
+
+
+def delta_state_size(n_heads: int, key_dim: int, value_dim: int) -> int:
+    """Floats of a request's matrices: [head][value column][padded key size]."""
+    r, lanes = delta_plan(key_dim)
+    return n_heads * value_dim * r * lanes
+
+
+def delta_state_matrix(state: torch.Tensor, n_heads: int, key_dim: int,
+                       value_dim: int) -> torch.Tensor:
+    """The matrices S [slots, H, d, dv] that the leading part of state rows holds (a copy)."""
+    r, lanes = delta_plan(key_dim)
+    P = r * lanes
+    m = state[:, :n_heads * value_dim * P].reshape(state.shape[0], n_heads, value_dim, P)
+    return m[..., :key_dim].transpose(2, 3).contiguous()
+
+
+@_launches("norm_rope_write")
+def short_conv(src: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, state_offset: int,
+               state_slots: torch.Tensor, seq_index: torch.Tensor, q_start: torch.Tensor,
+               out: torch.Tensor, unit_heads: int = 0, head_dim: int = 1, scaled_heads: int = 0,
+               scale: float = 1.0, unit_eps: float = 0.0, single_tokens: bool = False) -> None:
+    """out[t, c] = silu(sum_j taps[c, j] * x_(t - n + 1 + j)[c]) over the rows of a step: ``src``
+    [T, >= C] (contiguous rows, any row stride), ``taps`` float32 [C, n] (the last column is the
+    token's own), ``out`` float32 [T, C].  Rows before a sequence's portion come from its state:
+    [n - 1, C] floats from ``state_offset`` on in row state_slots[s] of ``state`` (float32
+    [slots, width]), oldest first; zeros for a new request.  After the step the state holds the
+    last n - 1 rows seen.  The leading ``unit_heads`` * ``head_dim`` channels are heads that
+    leave as unit vectors x / sqrt(sum x^2 + unit_eps), the first ``scaled_heads`` of them times
+    ``scale``.  ``single_tokens``: every sequence brings one token (one launch instead of two)."""
+    _need_gpu(taps, state, state_slots, seq_index, q_start, out)
+    if not src.is_cuda:
+        raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    for t, name in ((state_slots, "state_slots"), (seq_index, "seq_index"), (q_start, "q_start")):
+        _i32(t, name)
+    T = src.shape[0]
+    C, n = taps.shape
+    n_seqs = state_slots.shape[0]
+    if taps.dtype != torch.float32 or not taps.is_contiguous() or src.shape[1] < C \
+            or out.shape != (T, C) or out.dtype != torch.float32 or not out.is_contiguous() \
+            or state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 \
+            or state_offset < 0 or state_offset + (n - 1) * C > state.shape[1] \
+            or seq_index.shape[0] != T or q_start.shape[0] != n_seqs + 1 \
+            or unit_heads < 0 or head_dim < 1 or unit_heads * head_dim > C \
+            or scaled_heads > unit_heads or (single_tokens and T != n_seqs):
+        raise KernelUnavailable(f"short_conv: src {tuple(src.shape)}, taps {tuple(taps.shape)} "
+                                f"{taps.dtype}, out {tuple(out.shape)} {out.dtype}, state "
+                                f"{tuple(state.shape)} from {state_offset}")
+    lib = build.load("delta")
+    _check(lib.zf_short_conv(_ptr(src), _dt(src), ctypes.c_longlong(_columns(src, "short_conv: src")),
+                             _ptr(taps), n, _ptr(state), ctypes.c_longlong(state.stride(0)),
+                             ctypes.c_longlong(state_offset), _ptr(state_slots), _ptr(seq_index),
+                             _ptr(q_start), _ptr(out), T, n_seqs, C, int(unit_heads),
+                             int(head_dim), int(scaled_heads), ctypes.c_float(scale),
+                             ctypes.c_float(unit_eps), 1 if single_tokens else 0, _stream()),
+           "short_conv")
+
+
+@_launches("attention")
+def delta_recurrence(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, ab: torch.Tensor,
+                     decay_log: torch.Tensor, decay_bias: torch.Tensor, state: torch.Tensor,
+                     state_slots: torch.Tensor, q_start: torch.Tensor, out: torch.Tensor,
+                     n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int) -> None:
+    """The gated delta rule a head, token by token in 32-bit, over the rows of a step:
+    S <- g S; w = beta (v - S^T k); S <- S + k w^T; o = S^T q.  ``qkv`` float32 [T, C] holds
+    ``n_kv_heads`` q heads of ``key_dim`` from column q_off, as many k heads from k_off and
+    ``n_heads`` v heads of ``value_dim`` from v_off (value head n reads q/k head
+    floor(n / (n_heads / n_kv_heads))); ``ab`` float32 [T, 2 H]: z_a, then z_b, with
+    g = exp(-exp(decay_log) * softplus(z_a + decay_bias)) and beta = sigmoid(z_b)
+    (``decay_log``, ``decay_bias`` float32 [H]).  ``out`` float32 [T, H * dv].  Sequence s owns
+    the rows q_start[s] .. q_start[s + 1] - 1; its matrices (the leading ``delta_state_size``
+    floats of row state_slots[s] of ``state``) are read before its first row and written behind
+    its last.  A row's result depends on the state and the rows of its own sequence alone."""
+    _need_gpu(qkv, ab, decay_log, decay_bias, state, state_slots, q_start, out)
+    _i32(state_slots, "state_slots")
+    _i32(q_start, "q_start")
+    T, C = qkv.shape
+    H, KH, d, dv = int(n_heads), int(n_kv_heads), int(key_dim), int(value_dim)
+    n_seqs = state_slots.shape[0]
+    if not 0 < d <= DELTA_MAX_KEY_DIM or H < 1 or KH < 1 or H % KH != 0 or dv < 1:
+        raise KernelUnavailable(f"delta_recurrence: {H} heads on {KH} of {d} x {dv} (key size up "
+                                f"to {DELTA_MAX_KEY_DIM})")
+    r, lanes = delta_plan(d)
+    need = H * dv * r * lanes
+    if qkv.dtype != torch.float32 or not qkv.is_contiguous() or min(q_off, k_off, v_off) < 0 \
+            or max(q_off, k_off) + KH * d > C or v_off + H * dv > C \
+            or ab.shape != (T, 2 * H) or ab.dtype != torch.float32 or not ab.is_contiguous() \
+            or decay_log.shape != (H,) or decay_bias.shape != (H,) \
+            or decay_log.dtype != torch.float32 or decay_bias.dtype != torch.float32 \
+            or out.shape != (T, H * dv) or out.dtype != torch.float32 or not out.is_contiguous() \
+            or state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < need \
+            or state.stride(1) != 1 or state.stride(0) % 4 != 0 or state.data_ptr() % 16 != 0 \
+            or q_start.shape[0] != n_seqs + 1:
+        raise KernelUnavailable(f"delta_recurrence: qkv {tuple(qkv.shape)} {qkv.dtype}, ab "
+                                f"{tuple(ab.shape)}, out {tuple(out.shape)}, state "
+                                f"{tuple(state.shape)} (rows a multiple of 4 floats, at least "
+                                f"{need})")
+    # a workgroup: whole waves, at most 256 threads, no more columns than the head has
+    cols = min(256, (dv * lanes + 63) // 64 * 64) // lanes
+    lib = build.load("delta")
+    _check(lib.zf_delta_recurrence(_ptr(qkv), C, int(q_off), int(k_off), int(v_off), _ptr(ab),
+                                   _ptr(decay_log), _ptr(decay_bias), _ptr(state),
+                                   ctypes.c_longlong(state.stride(0)), _ptr(state_slots),
+                                   _ptr(q_start), _ptr(out), n_seqs, H, KH, d, dv, r, lanes, cols,
+                                   _stream()), "delta_recurrence")

@@ -25,7 +25,7 @@ from ..errors import KernelUnavailable
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 MODULES = ("elementwise", "gemm", "attention", "sampling", "randinit", "norms",
-           "sink_attention", "moe", "masked_attention", "recurrent")
+           "sink_attention", "moe", "masked_attention", "recurrent", "delta")
 HOST_MODULES = ("cache_core",)
 HEADERS = ("zf_common.h", "zf_no_alloc.h")
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]

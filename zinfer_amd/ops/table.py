@@ -10,6 +10,7 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from . import (gated_act, moe_grouped, norm_add_norm, tied_attention_mfma)
+from . import delta_recurrence, short_conv, streams_step
 from . import (concat_rows, decay_recurrence, embed_sinusoid, head_norm_gate, token_shift_mix)
 from . import (activation, head_products, masked_attention, masked_attention_mfma,
                norm_add_store, project_rows)
@@ -110,6 +111,13 @@ KERNELS: Dict[str, KernelEntry] = {
                                     "a key channel and grown by k v^T, token by token"),
     "head_norm_gate": KernelEntry(head_norm_gate, "recurrent", "own: RMS norm a head, gain and "
                                   "silu gate"),
+    "streams_step": KernelEntry(streams_step, "norms", "own: a residual stream in several "
+                                "copies: a sublayer's output joins them, the next one's input "
+                                "is read from them and normed"),
+    "short_conv": KernelEntry(short_conv, "delta", "own: causal convolutions over time a channel "
+                              "with silu and unit heads, the last rows kept as state"),
+    "delta_recurrence": KernelEntry(delta_recurrence, "delta", "own: a matrix a head, decayed "
+                                    "and corrected towards every token's value"),
     "mfma_loop": KernelEntry(mfma_loop, "gemm",
                              "own: MFMAs alone, the rate the tiled products are measured against"),
 }

@@ -2,4 +2,4 @@ from .base import (Block, BuildContext, FeedForward, KVNeed, Mixer, Norm, Part,
                    PositionEncoding, StateNeed, StepHints, StepShape, TensorDecl, build_part,
                    register_part, unregister_part)
 from .linear import Linear, place_gain, place_matrix
-from . import norm, position, attention, tied_attention, masked_attention, recurrent, mlp, moe, block  # registers the built-in parts
+from . import norm, position, attention, tied_attention, masked_attention, recurrent, delta, mlp, moe, block  # registers the built-in parts

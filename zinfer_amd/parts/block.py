@@ -5,8 +5,10 @@ from typing import Dict
 import torch
 
 from ..config.specs import (ParallelBlockSpec, PostNormBlockSpec, PreNormBlockSpec,
-                            SandwichNormBlockSpec)
+                            SandwichNormBlockSpec, StreamBlockSpec)
+from ..errors import ConfigError
 from .base import Block, TensorDecl, build_part, register_part
+from .linear import place_gain
 
 
 class PreNormBlock(Block):
@@ -323,6 +325,153 @@ class ParallelBlock(Block):
         step.norm_ready = step.norm_after = None
 
 
+class StreamRead:
+    """What the kernel that last wrote the copies ``x`` of the stream left for the block that
+    reads them next: the rows ``normed`` its first sublayer takes."""
+
+    def __init__(self, block, x: torch.Tensor, normed: torch.Tensor):
+        self.block, self.x, self.normed = block, x, normed
+
+    def fits(self, block, x: torch.Tensor) -> bool:
+        return self.block is block and self.x.data_ptr() == x.data_ptr() \
+            and self.x.shape == x.shape
+
+
+class StreamBlock(Block):
+    """A layer over several copies of the residual stream (``StreamBlockSpec``): x is float32
+    [S, T, W] (or [T, W] for one copy).  One kernel a sublayer: it lets the sublayer before join
+    every copy (the copies mixed among themselves, the output added with a weight a copy) and
+    forms the next sublayer's input, the weighted sum of the new copies through the norm.  That
+    holds across layers too: the last kernel of a block already reads for the block behind it
+    (``StreamRead`` in ``step.norm_ready``), which the decoder names in
+    ``step.norm_after_block``.  A sublayer stores its output in a float32 branch; a mixer that
+    is two side by side may bring two branches with a factor each (``forward_branches``), which
+    the same kernel adds.  The norms' work is done by that kernel: they must be RMS norms
+    without a bias (``LayerNormSpec`` not centred)."""
+
+    def __init__(self, spec: StreamBlockSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        from .. import ops
+        if not 1 <= spec.streams <= ops.STREAMS_MAX:
+            raise ConfigError(f"streams={spec.streams}: 1 to {ops.STREAMS_MAX} copies of the "
+                              "residual stream")
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx, prefix + spec.mixer_norm_prefix)
+        self.mixer = build_part("mixer", spec.mixer, ctx, prefix + spec.mixer_prefix)
+        self.parts = [self.mixer_norm, self.mixer]
+        self.ff_norm = self.feed_forward = None
+        if spec.feed_forward is not None:
+            self.ff_norm = build_part("norm", spec.ff_norm, ctx, prefix + spec.ff_norm_prefix)
+            self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
+                                           prefix + spec.ff_prefix)
+            self.parts += [self.ff_norm, self.feed_forward]
+        self.parts = tuple(self.parts)
+        for norm in (self.mixer_norm, self.ff_norm):
+            ns = getattr(norm, "spec", None)
+            if norm is not None and (getattr(ns, "centred", True) or
+                                     getattr(ns, "bias_name", "") is not None):
+                raise ConfigError("the norms of a layer over several copies of the stream are "
+                                  "RMS norms without a bias")
+        # the block that runs before this one may read the copies for it
+        self.entry_norm = self
+        self.defers = False
+        self.graph_safe = all(p.graph_safe for p in self.parts)
+        self.kernel_modules = tuple(sorted({"norms"}
+                                           | {m for p in self.parts for m in p.kernel_modules}))
+
+    def _coef_names(self, c: int):
+        s = self.spec
+        base = self.prefix + s.coef_prefix.format(c)
+        return base + s.in_name, base + s.mix_name, base + s.out_name
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        d: Dict[str, TensorDecl] = {}
+        for part in self.parts:
+            d.update(part.declare())
+        S = self.spec.streams
+        if self.spec.learned:
+            for c in (1, 2) if self.feed_forward is not None else (1,):
+                a, m, b = self._coef_names(c)
+                d[a] = TensorDecl((S,), init="gain")
+                d[m] = TensorDecl((S, S))
+                d[b] = TensorDecl((S,), init="gain")
+        return d
+
+    def bind(self, tensors) -> None:
+        for part in self.parts:
+            part.bind(tensors)
+        S = self.spec.streams
+        self.coefs = []
+        for c in (1, 2) if self.feed_forward is not None else (1,):
+            if self.spec.learned:
+                a, m, b = (place_gain(tensors[n], self.ctx) for n in self._coef_names(c))
+            else:
+                a, b = (place_gain(torch.ones(S), self.ctx) for _ in range(2))
+                m = place_gain(torch.eye(S), self.ctx)
+            self.coefs.append((a, m, b))
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def accept_cache(self, cache) -> None:
+        self.mixer.accept_cache(cache)
+
+    def hint_providers(self):
+        return [q for p in self.parts for q in p.hint_providers()]
+
+    def read_args(self, c: int = 0):
+        """What the kernel that reads the copies for sublayer ``c`` needs."""
+        norm = self.mixer_norm if c == 0 else self.ff_norm
+        return dict(in_coef=self.coefs[c][0], gain=norm.gain, eps=float(norm.spec.eps))
+
+    def _run(self, part, h, step, args):
+        """The sublayer's output as [(float32 branch, factor)]."""
+        branches = getattr(part, "forward_branches", None)
+        if branches is not None:
+            return branches(h, step, *args)
+        y = step.scratch("branch", h.shape, torch.float32)
+        if getattr(part, "stores_output", False):
+            part.forward(h, y, step, *args, accumulate=False)
+        else:
+            y.zero_()
+            part.forward(h, y, step, *args)
+        return [(y, 1.0)]
+
+    def forward(self, x, step, cache) -> None:
+        from .. import ops
+        xs = x if x.dim() == 3 else x.unsqueeze(0)
+        T, W = xs.shape[1], xs.shape[2]
+        act = self.ctx.act_dtype
+        after = step.norm_after_block
+        left, step.norm_ready, step.norm_after = step.norm_ready, None, None
+        if isinstance(left, StreamRead) and left.fits(self, x):
+            h = left.normed
+        else:
+            h = step.scratch("normed", (T, W), act)
+            ops.streams_step(xs, read=True, out=h, **self.read_args(0))
+        sublayers = [(self.mixer, (cache,))]
+        if self.feed_forward is not None:
+            sublayers.append((self.feed_forward, ()))
+        handed = None
+        for c, (part, args) in enumerate(sublayers):
+            branches = self._run(part, h, step, args)
+            _, mix, out_coef = self.coefs[c]
+            if c + 1 < len(sublayers):
+                reader = self.read_args(c + 1)
+            else:
+                reader = after.read_args(0) if isinstance(after, StreamBlock) else None
+            if reader is not None:
+                # (the sublayer is done with the buffer its input lay in)
+                h = step.scratch("normed_ff" if c % 2 == 0 else "normed", (T, W), act)
+                ops.streams_step(xs, branches, mix, out_coef, read=True, out=h, **reader)
+                if c + 1 == len(sublayers):
+                    handed = StreamRead(after, x, h)
+            else:
+                ops.streams_step(xs, branches, mix, out_coef)
+        step.norm_after = None
+        step.norm_ready = handed
+
+
+register_part("block", StreamBlockSpec, StreamBlock)
 register_part("block", ParallelBlockSpec, ParallelBlock)
 register_part("block", PostNormBlockSpec, PostNormBlock)
 register_part("block", PreNormBlockSpec, PreNormBlock)

@@ -64,8 +64,13 @@ class MaskedGqaAttention(Mixer):
              p + s.v_name: TensorDecl((self.v_width, s.hidden_size)),
              p + s.o_name: TensorDecl((s.hidden_size, s.n_heads * s.value_dim))}
         if s.qk_norm_eps is not None:
-            d[p + s.q_norm_name] = TensorDecl((self.q_width,), init="gain")
-            d[p + s.k_norm_name] = TensorDecl((self.k_width,), init="gain")
+            per = s.qk_norm_per_head
+            d[p + s.q_norm_name] = TensorDecl((s.head_dim if per else self.q_width,), init="gain")
+            d[p + s.k_norm_name] = TensorDecl((s.head_dim if per else self.k_width,), init="gain")
+        if s.bias:
+            for name, width in ((s.q_name, self.q_width), (s.k_name, self.k_width),
+                                (s.v_name, self.v_width)):
+                d[p + name + s.bias_suffix] = TensorDecl((width,))
         if s.sink:
             d[p + s.sink_name] = TensorDecl((s.n_heads,))
         if s.head_gate:
@@ -82,6 +87,11 @@ class MaskedGqaAttention(Mixer):
         self.proj = Linear(place_matrix(torch.cat(rows, dim=0), self.ctx))
         self.o = Linear(place_matrix(tensors[p + s.o_name], self.ctx))
         self.q_gain = self.k_gain = self.sink = None
+        self.q_bias = self.k_bias = self.v_bias = None
+        if s.bias:
+            self.q_bias, self.k_bias, self.v_bias = (
+                place_gain(tensors[p + n + s.bias_suffix], self.ctx)
+                for n in (s.q_name, s.k_name, s.v_name))
         if s.qk_norm_eps is not None:
             self.q_gain = place_gain(tensors[p + s.q_norm_name], self.ctx)
             self.k_gain = place_gain(tensors[p + s.k_norm_name], self.ctx)
@@ -109,16 +119,19 @@ class MaskedGqaAttention(Mixer):
         self.proj.forward(h, proj)
         q = step.scratch("q", (T, self.q_width), act)
         eps = float(s.qk_norm_eps) if s.qk_norm_eps is not None else 0.0
-        rot = dict(rot_dims=s.rotary.dims, freq=self.freq, mag=s.rotary.magnitude) \
-            if s.rotary is not None else {}
+        rot = dict(rot_dims=s.rotary.dims, freq=self.freq, mag=s.rotary.magnitude,
+                   interleaved=s.rotary.interleaved) if s.rotary is not None else {}
+        per = dict(per_head=s.qk_norm_per_head)
         segments = [ops.RowSegment(0, self.q_width, q, gain=self.q_gain, eps=eps, hd=s.head_dim,
-                                   **rot)]
+                                   bias=self.q_bias, **per, **rot)]
         if cache.writes:
             segments.append(ops.RowSegment(self.q_width, self.k_width, cache.k_pool,
                                            gain=self.k_gain, eps=eps, hd=s.head_dim,
-                                           pool_heads=s.n_kv_heads, **rot))
+                                           pool_heads=s.n_kv_heads, bias=self.k_bias, **per,
+                                           **rot))
             segments.append(ops.RowSegment(self.q_width + self.k_width, self.v_width, cache.v_pool,
-                                           hd=s.value_dim, pool_heads=s.n_kv_heads))
+                                           hd=s.value_dim, pool_heads=s.n_kv_heads,
+                                           bias=self.v_bias))
         ops.project_rows(proj, step.positions, kv.slot_mapping if cache.writes else None,
                          cache.page_size, segments)
         gate = proj[:, self.q_width + self.k_width + self.v_width:] if s.head_gate else None

@@ -22,13 +22,13 @@ class SwiGluMlp(FeedForward):
 
     def declare(self) -> Dict[str, TensorDecl]:
         s, p = self.spec, self.prefix
-        return {p + "gate_proj.weight": TensorDecl((s.intermediate_size, s.hidden_size)),
-                p + "up_proj.weight": TensorDecl((s.intermediate_size, s.hidden_size)),
-                p + "down_proj.weight": TensorDecl((s.hidden_size, s.intermediate_size))}
+        return {p + s.gate_name: TensorDecl((s.intermediate_size, s.hidden_size)),
+                p + s.up_name: TensorDecl((s.intermediate_size, s.hidden_size)),
+                p + s.down_name: TensorDecl((s.hidden_size, s.intermediate_size))}
 
     def bind(self, tensors) -> None:
-        p = self.prefix
-        g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
+        s, p = self.spec, self.prefix
+        g, u = tensors[p + s.gate_name], tensors[p + s.up_name]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         g, u = place_matrix(g, self.ctx), place_matrix(u, self.ctx)
@@ -39,7 +39,7 @@ class SwiGluMlp(FeedForward):
         stacked = ops.interleave_gate_up(g, u) if self.fused else torch.cat([g, u], dim=0)
         del g, u
         self.gate_up = Linear(stacked)
-        self.down = Linear(place_matrix(tensors[p + "down_proj.weight"], self.ctx))
+        self.down = Linear(place_matrix(tensors[p + s.down_name], self.ctx))
 
     def forward(self, h, residual, step) -> None:
         T = h.shape[0]

@@ -135,7 +135,8 @@ class LayerNorm(Norm):
 
     def declare(self) -> Dict[str, TensorDecl]:
         s = self.spec
-        d = {self.prefix + s.weight_name: TensorDecl((s.width,), init="gain")}
+        d = {self.prefix + s.weight_name: TensorDecl(
+            (s.width,), init="gain" if s.gain_offset == 0.0 else "normal")}
         if s.bias_name is not None:
             d[self.prefix + s.bias_name] = TensorDecl((s.width,))
         return d
@@ -143,6 +144,10 @@ class LayerNorm(Norm):
     def bind(self, tensors) -> None:
         s = self.spec
         self.gain = place_gain(tensors[self.prefix + s.weight_name], self.ctx)
+        if s.gain_offset != 0.0:
+            # a weight stored around zero: the gain is the offset plus the weight, added once
+            # in 32-bit
+            self.gain = (self.gain + float(s.gain_offset)).contiguous()
         self.bias = place_gain(tensors[self.prefix + s.bias_name], self.ctx) \
             if s.bias_name is not None else None
 
