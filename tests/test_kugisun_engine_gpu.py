@@ -229,7 +229,7 @@ def test_every_run_of_a_layer_alone():
         assert len(seen) == len(sums)
         for pos, (got, want) in enumerate(zip(seen, sums)):
             err = float((got - want).abs().max() / want.abs().max())
-            assert err < 2e-5, f"{name} run {pos}: {err:.3g}"
+            assert err < TOL["float32"], f"{name} run {pos}: {err:.3g}"
 
 
 def _loud(name, which):

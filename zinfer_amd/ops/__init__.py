@@ -1855,10 +1855,11 @@ def gated_act(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: flo
     """out[t, j] = g * sigmoid(alpha g) * (u + shift) with g = min(gate_up[t, j], limit) and
     u = clamp(gate_up[t, ff + j], -limit, limit) (no clamp if limit <= 0); times
     ``row_factor[t]`` (float32 [T] or a column of a float32 matrix) if given."""
-    _need_gpu(gate_up, out, row_factor)
+    _need_gpu(gate_up, out)
     T, ff = out.shape
     if gate_up.shape != (T, 2 * ff) or gate_up.dtype != out.dtype \
-            or (row_factor is not None and (row_factor.dtype != torch.float32
+            or (row_factor is not None and (not row_factor.is_cuda
+                                            or row_factor.dtype != torch.float32
                                             or row_factor.dim() != 1 or row_factor.shape[0] != T)):
         raise KernelUnavailable(f"gated_act: gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)}")
     lib = build.load("moe")
