@@ -163,6 +163,9 @@ TESTED_AGAINST = {
     "token_shift_mix": "plain_nupovik.py:token_shift",
     "decay_recurrence": "plain_nupovik.py:decayed_outer_recurrence",
     "head_norm_gate": "test_nupovik_kernels_gpu.py:test_head_norm_gate",
+    "streams_step": "plain_kugisun.py:stream_step",
+    "short_conv": "plain_kugisun.py:short_convolution",
+    "delta_recurrence": "plain_kugisun.py:delta_rule",
 }
 
 
