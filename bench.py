@@ -23,7 +23,7 @@ intermediate 25600; 65.5 GB of weights): a 2048-token prefill, then decode at ba
 64 with every request's context just below 8192 tokens; the cache pool is sized for
 64 x 8192 tokens (137 GB).
 
-``--workload fezupel``, ``--workload lodenex`` and ``--workload nupovik``: shapes of those three
+``--workload fezupel``, ``--workload lodenex``, ``--workload nupovik`` and ``--workload kugisun``: shapes of those
 designs at layer sizes that resemble served models, each beside the dense Qwen3 decoder of equal
 size (prefill of 2048 tokens, decode at batch 8), and their kernels alone beside the like
 kernels of that decoder.
@@ -1286,11 +1286,323 @@ def main_nupovik(args) -> int:
         "shapes": shapes}))
     return 0
 
+# --------------------------------------------------------------------------- Kugisun beside Qwen3
+# Layer sizes that resemble served models of this kind: a stream in four copies, attention heads
+# of 128 beside delta-rule heads of 128 x 128, a gated feed-forward or a mixture with outputs
+# that hand their input on and a shared expert.  Every shape is run beside the dense Qwen3
+# decoder of the same width, depth and vocabulary whose attention has the left mixer's heads and
+# whose gated feed-forward does the matrix work a token of the new design's feed-forwards; the
+# new kernels alone stand beside the like kernels of that decoder and of Nupovik, the closest
+# design with a recurrence (its gated linear attention at the same heads).
+def _kg_moe(experts, identity, top, ff, groups, shared):
+    return {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": shared},
+            "router": {"experts": experts, "identity": identity, "top": top, "scale": 2.0,
+                       "groups": {"count": groups[0], "keep": groups[1]}}}
+
+
+def _kg_mixer(heads, kv, r_heads, r_kv):
+    return {"left": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128,
+                     "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 500000.0}},
+            "right": {"heads": r_heads, "kv_heads": r_kv, "dim": 128, "vdim": 128, "conv": 4},
+            "left_scale": 0.8, "right_scale": 0.9}
+
+
+KUGISUN_SHAPES = {
+    "medium": dict(width=2048, vocab=32768, streams=4, mixer=_kg_mixer(16, 4, 16, 8),
+                   mlps=[{"kind": "dense", "ff": 5632}, _kg_moe(30, 2, 4, 1024, (8, 4), 1536)],
+                   order=[0, 1, 1, 1]),
+    "wide": dict(width=4096, vocab=32768, streams=4, mixer=_kg_mixer(32, 8, 32, 16),
+                 mlps=[{"kind": "dense", "ff": 11264}, _kg_moe(62, 2, 6, 1536, (8, 4), 2048)],
+                 order=[0, 1, 0, 1]),
+}
+
+
+def kugisun_config(sh: dict, max_positions: int) -> dict:
+    layers, first = [], {}
+    for i, j in enumerate(sh["order"]):
+        L = {"type": "parallel", "mixer": sh["mixer"], "mlp": sh["mlps"][j]}
+        if j in first:
+            L["weights_of"] = first[j]
+        first.setdefault(j, i)
+        layers.append(L)
+    return {"architecture": "Kugisun", "vocab": sh["vocab"], "width": sh["width"],
+            "max_positions": max_positions, "streams": sh["streams"], "norm": {"eps": 1e-6},
+            "layers": layers}
+
+
+def _kg_used(mlp: dict) -> int:
+    return mlp["ff"] if mlp["kind"] == "dense" \
+        else mlp["router"]["top"] * mlp["expert"]["ff"] + mlp["shared"]["ff"]
+
+
+def kugisun_twin(sh: dict, max_positions: int) -> dict:
+    used = [_kg_used(sh["mlps"][j]) for j in sh["order"]]
+    left = sh["mixer"]["left"]
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+                num_hidden_layers=len(sh["order"]), hidden_size=sh["width"],
+                num_attention_heads=left["heads"], num_key_value_heads=left["kv_heads"],
+                head_dim=128, intermediate_size=int(sum(used) / len(used)) // 64 * 64,
+                vocab_size=sh["vocab"], rope_theta=1000000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=True, max_position_embeddings=max_positions,
+                torch_dtype="bfloat16")
+
+
+def kugisun_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float) -> dict:
+    """The new design's kernels alone beside the like kernels of the dense decoder and of
+    Nupovik, at ``T`` tokens of one sequence that holds ``ctx`` tokens (T = ctx: a prompt;
+    T = 1 x 8 sequences: a decode step), each with the fraction of its bound it reaches: matrix
+    work against the MFMA loop's rate (prompt) or the bytes that must be read against the
+    measured read stream (decode); the recurrences are 32-bit vector work (the delta rule six
+    operations a state element a token, the decayed sum five) against the published 32-bit
+    vector rate, or their state read and written once (decode)."""
+    import torch
+    import zinfer_amd.ops as ops
+    dev = "cuda:0"
+    W, S = sh["width"], sh["streams"]
+    left, right = sh["mixer"]["left"], sh["mixer"]["right"]
+    bf = torch.bfloat16
+    decode = T == 1
+    n_seqs = 8 if decode else 1
+    rows = n_seqs * T
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev) * 0.05).to(bf)
+    rnd32 = lambda *shape: torch.randn(shape, generator=g, device=dev) * 0.05
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)
+    pages = (ctx + PAGE - 1) // PAGE
+    table = torch.arange(n_seqs * pages, dtype=torch.int32, device=dev).view(n_seqs, pages)
+    q_start = i32([i * T for i in range(n_seqs + 1)])
+    ctx_len = i32([ctx] * n_seqs)
+    seq_index = i32([i for i in range(n_seqs) for _ in range(T)])
+    positions = i32([ctx - T + i for _ in range(n_seqs) for i in range(T)])
+    slot_mapping = i32([s * pages * PAGE + ctx - T + i for s in range(n_seqs) for i in range(T)])
+    state_slots = i32(list(range(n_seqs)))
+    out = {}
+
+    def row(name, t_new, work_new, rate_new, bound_new, like=None, t_old=None, work_old=None,
+            rate_old=None, bound_old=None):
+        r = {"kugisun_us": round(t_new * 1e6, 1),
+             "kugisun_frac_of_" + bound_new: round(work_new / t_new / rate_new, 4)}
+        if t_old is not None:
+            r.update({"like": like, "like_us": round(t_old * 1e6, 1),
+                      "like_frac_of_" + bound_old: round(work_old / t_old / rate_old, 4)})
+        out[name] = r
+
+    mat_bound, mat_rate = ("read", read_bw) if decode else ("mfma", mfma_rate)
+    # ---- attention: the masked kernels at the left mixer's heads beside the dense decoder's
+    nH, nKV, hd = left["heads"], left["kv_heads"], 128
+    q = rnd(rows, nH * hd)
+    k_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    v_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    o = torch.empty((rows, nH * hd), dtype=bf, device=dev)
+    t_old = _timed_graph(lambda: ops.paged_attention(q, k_pool, v_pool, table, q_start, ctx_len,
+                                                     seq_index, o, hd ** -0.5, 0, nH, nKV, hd,
+                                                     PAGE, T, ctx))
+    t_new = _timed_graph(lambda: ops.attend_masked(q, None, None, k_pool, v_pool, None, table,
+                                                   q_start, ctx_len, seq_index, o, hd ** -0.5, 0.0,
+                                                   0, 0, nH, nKV, hd, hd, PAGE, T, ctx))
+    pairs = n_seqs * (ctx if decode else T * (T + 1) // 2)
+    att_work = n_seqs * ctx * nKV * 2 * hd * 2 if decode else 4.0 * pairs * hd * nH
+    row("attention", t_new, att_work, mat_rate, mat_bound, "qwen3 attention", t_old, att_work,
+        mat_rate, mat_bound)
+    # ---- bias, norm a head, rotation, cache write beside the dense decoder's kernel
+    qkv = rnd(rows, (nH + 2 * nKV) * hd)
+    bias = rnd32((nH + 2 * nKV) * hd)
+    gq, gk = torch.ones(hd, device=dev), torch.ones(hd, device=dev)
+    freq = torch.tensor([500000.0 ** (-2.0 * i / 64) for i in range(32)], device=dev)
+    qw, kw = nH * hd, nKV * hd
+    segs = [ops.RowSegment(0, qw, o, gain=gq, eps=1e-6, hd=hd, bias=bias[:qw].contiguous(),
+                           per_head=True, rot_dims=64, freq=freq, interleaved=True),
+            ops.RowSegment(qw, kw, k_pool, gain=gk, eps=1e-6, hd=hd, pool_heads=nKV,
+                           bias=bias[qw:qw + kw].contiguous(), per_head=True, rot_dims=64,
+                           freq=freq, interleaved=True),
+            ops.RowSegment(qw + kw, kw, v_pool, hd=hd, pool_heads=nKV,
+                           bias=bias[qw + kw:].contiguous())]
+    t_new = _timed_graph(lambda: ops.project_rows(qkv, positions, slot_mapping, PAGE, segs))
+    cos = torch.ones((ctx + 1, hd // 2), device=dev)
+    sin = torch.zeros((ctx + 1, hd // 2), device=dev)
+    kp2 = torch.empty_like(k_pool)
+    vp2 = torch.empty_like(v_pool)
+    t_old = _timed_graph(lambda: ops.qk_norm_rope_kv_write(qkv, gq, gk, 1e-6, cos, sin, positions,
+                                                           slot_mapping, kp2, vp2, o, nH, nKV, hd,
+                                                           PAGE))
+    rw = rows * (nH + 2 * nKV) * hd * 2 * 2
+    row("norm_rotate_write", t_new, rw, read_bw, "read", "qwen3 norm, rotation, cache write",
+        t_old, rw, read_bw, "read")
+    # ---- the delta rule beside Nupovik's decayed sum at the same heads
+    H, KH, d, dv, taps = right["heads"], right["kv_heads"], right["dim"], right["vdim"], right["conv"]
+    C = 2 * KH * d + H * dv
+    msize = (ops.delta_state_size(H, d, dv) + 3) // 4 * 4
+    state = torch.zeros((n_seqs, msize + (taps - 1) * C), dtype=torch.float32, device=dev)
+    f32qkv = rnd32(rows, C)
+    f32qkv[:, :2 * KH * d] = torch.nn.functional.normalize(
+        f32qkv[:, :2 * KH * d].view(rows, 2 * KH, d), dim=-1).view(rows, -1)
+    ab = torch.randn((rows, 2 * H), generator=g, device=dev)
+    a_log, dtb = torch.zeros(H, device=dev) - 3.0, torch.zeros(H, device=dev)
+    ro = torch.empty((rows, H * dv), dtype=torch.float32, device=dev)
+    t_new = _timed_graph(lambda: ops.delta_recurrence(f32qkv, 0, KH * d, 2 * KH * d, ab, a_log,
+                                                      dtb, state, state_slots, q_start, ro, H, KH,
+                                                      d, dv))
+    size = ops.recurrence_state_size(H, d, dv)
+    st2 = torch.zeros((n_seqs, size), dtype=torch.float32, device=dev)
+    qk = rnd(2, rows, H * d)
+    v = rnd(rows, H * dv)
+    z = torch.randn((rows, H * d), generator=g, device=dev)
+    zb = torch.zeros((H * d,), device=dev)
+    t_old = _timed_graph(lambda: ops.decay_recurrence(qk[0], qk[1], v, z, zb, None, st2,
+                                                      state_slots, q_start, ro, H, d, dv,
+                                                      "sigmoid_root", tau=16.0, q_scale=d ** -0.5,
+                                                      max_q_len=T))
+    if decode:
+        sb = 2.0 * n_seqs * H * d * dv * 4
+        row("delta_recurrence", t_new, sb, read_bw, "read", "nupovik decayed sum", t_old, sb,
+            read_bw, "read")
+    else:
+        row("delta_recurrence", t_new, 6.0 * rows * H * d * dv, PEAK_FLOPS["fp32"], "fp32_vector",
+            "nupovik decayed sum", t_old, 5.0 * rows * H * d * dv, PEAK_FLOPS["fp32"],
+            "fp32_vector")
+    # ---- short convolutions beside Nupovik's token shift (both read rows and a kept row)
+    proj = rnd(rows, C + H * dv)
+    tapw = torch.randn((C, taps), generator=g, device=dev)
+    cout = torch.empty((rows, C), dtype=torch.float32, device=dev)
+    t_new = _timed_graph(lambda: ops.short_conv(proj, tapw, state, msize, state_slots, seq_index,
+                                                q_start, cout, unit_heads=2 * KH, head_dim=d,
+                                                scaled_heads=KH, scale=d ** -0.5, unit_eps=1e-6,
+                                                single_tokens=decode))
+    hrow = rnd(rows, W)
+    mu = torch.rand((5, W), generator=g, device=dev)
+    mixes = torch.empty((5, rows, W), dtype=bf, device=dev)
+    st3 = torch.zeros((n_seqs, W), dtype=torch.float32, device=dev)
+    t_old = _timed_graph(lambda: ops.token_shift_mix(hrow, mu, st3, 0, state_slots, seq_index,
+                                                     q_start, mixes))
+    row("short_conv", t_new, rows * C * (2 + 4), read_bw, "read", "nupovik token shift", t_old,
+        rows * W * 2 * (1 + 5), read_bw, "read")
+    gate = rnd(rows, H * dv)
+    gain = torch.ones((dv,), device=dev)
+    mixed = torch.empty((rows, H * dv), dtype=bf, device=dev)
+    t_norm = _timed_graph(lambda: ops.head_norm_gate(ro, gain, gate, mixed, H, 1e-6))
+    row("head_norm_gate", t_norm, rows * H * dv * (4 + 2 + 2), read_bw, "read")
+    # ---- the copies: write and read in one launch beside the dense decoder's norm
+    x = torch.randn((S, rows, W), generator=g, device=dev)
+    y0, y1 = rnd32(rows, W), rnd32(rows, W)
+    M = torch.eye(S, device=dev) + 0.1 * torch.randn((S, S), generator=g, device=dev)
+    bco, aco = torch.ones(S, device=dev), torch.ones(S, device=dev) / S
+    gw = torch.ones(W, device=dev)
+    hout = torch.empty((rows, W), dtype=bf, device=dev)
+    t_new = _timed_graph(lambda: ops.streams_step(x, [(y0, 0.8), (y1, 1.0)], M, bco, read=True,
+                                                  in_coef=aco, gain=gw, eps=1e-6, out=hout))
+    x1 = torch.randn((rows, W), generator=g, device=dev)
+    t_old = _timed_graph(lambda: ops.rmsnorm(x1, gw, 1e-6, hout))
+    row("streams_step", t_new, rows * W * (4 * (2 * S + 2) + 2), read_bw, "read", "qwen3 norm",
+        t_old, rows * W * (4 + 2), read_bw, "read")
+    # ---- feed-forwards
+    h = rnd(rows, W)
+    branch = torch.zeros((rows, W), dtype=torch.float32, device=dev)
+
+    def gated(inter):
+        wgu = ops.pretile_weight(ops.interleave_gate_up(rnd(inter, W), rnd(inter, W)))
+        wd = ops.pretile_weight(rnd(W, inter))
+        act2 = torch.empty((rows, inter), dtype=bf, device=dev)
+
+        def run():
+            ops.gemm_swiglu(h, wgu, act2, w_tiled=True)
+            ops.gemm(act2, wd, branch, accumulate=True, w_tiled=True)
+        return _timed_graph(run)
+    moe = next(f for f in sh["mlps"] if f["kind"] == "moe")
+    r = moe["router"]
+    E, I, top, ff, shared = r["experts"], r["identity"], r["top"], moe["expert"]["ff"], moe["shared"]["ff"]
+    groups = (r["groups"]["count"], r["groups"]["keep"])
+    router = torch.randn((E + I + 1, W), generator=g, device=dev) * 0.05
+    correction = torch.randn((E + I,), generator=g, device=dev) * 0.01
+    ids = torch.empty((rows, top), dtype=torch.int32, device=dev)
+    share = torch.empty((rows, top), dtype=torch.float32, device=dev)
+    sgate = torch.empty((rows, 1), dtype=torch.float32, device=dev)
+    gu, down = rnd(E, 2 * ff, W), rnd(E, W, ff)
+    y = torch.empty((rows, top, ff), dtype=bf, device=dev)
+    wsgu = ops.pretile_weight(rnd(2 * shared, W))
+    wsd = ops.pretile_weight(rnd(W, shared))
+    sgu = torch.empty((rows, 2 * shared), dtype=bf, device=dev)
+    sy = torch.empty((rows, shared), dtype=bf, device=dev)
+
+    def mixture():
+        ops.moe_route(h, router, None, ids, share, scoring="softmax_all", correction=correction,
+                      groups=groups, group_mark=1, normalize=False, weight_scale=2.0, extra=sgate)
+        ops.moe_experts(h, gu, down, ids, share, y, branch, 0.0, 1.0, 0.0, add=False, n_identity=I)
+        ops.gemm(h, wsgu, sgu, w_tiled=True)
+        ops.gated_act(sgu, sy, 0.0, 1.0, 0.0, row_factor=sgate[:, 0])
+        ops.gemm(sy, wsd, branch, accumulate=True, w_tiled=True)
+    t_new = _timed_graph(mixture)
+    inter = (top * ff + shared) // 64 * 64
+    t_old = gated(inter)
+    if decode:
+        used = min(E, rows * top)
+        row("mixture", t_new, (used * ff + shared) * 3 * W * 2, read_bw, "read",
+            "qwen3 feed-forward of the width a token uses", t_old, 3 * inter * W * 2, read_bw,
+            "read")
+    else:
+        row("mixture", t_new, 2.0 * rows * 3 * (top * ff + shared) * W, mfma_rate, "mfma",
+            "qwen3 feed-forward of the width a token uses", t_old, 2.0 * rows * 3 * inter * W,
+            mfma_rate, "mfma")
+    return out
+
+
+def main_kugisun(args) -> int:
+    """Prefill and decode throughput of Kugisun shapes beside the dense Qwen3 decoder of equal
+    size, and the new kernels alone beside the like kernels of that decoder and of Nupovik."""
+    import torch
+    import zinfer_amd.ops as ops
+    from zinfer_amd.config import entry_for
+    T, batch, prompt = args.prefill_tokens, args.batch, args.prompt_len
+    max_positions = max(T, prompt + args.steps + args.warmup + 64) + 64
+    read_bw = ops.measure_read_bandwidth("cuda:0")
+    mfma_rate = ops.measure_mfma_rate("cuda:0")
+    names = [args.kugisun_shape] if args.kugisun_shape else list(KUGISUN_SHAPES)
+    shapes = {}
+    for name in names:
+        sh = KUGISUN_SHAPES[name]
+        row = {"sizes": {k: sh[k] for k in ("width", "vocab", "streams", "mixer", "mlps", "order")}}
+        for label, raw in (("kugisun", kugisun_config(sh, max_positions)),
+                           ("qwen3", kugisun_twin(sh, max_positions))):
+            cfg = entry_for(raw).config_type.from_dict(raw)
+            pool = batch * (prompt + args.steps + args.warmup + 64) + T + 256
+            llm = build_llm(raw, args.dtype, args.seed, pool, max(batch, 8),
+                            max_step_tokens=max(T, 2048), multi_step=args.multi_step)
+            t_pre = run_prefill(llm, cfg, T, args.seed + 1)
+            dt, mean_ctx = run_decode(llm, cfg, batch, prompt, args.steps, args.warmup, args.seed + 2)
+            row[label] = {"prefill_tokens_per_s": round(T / t_pre, 1), "prefill_ms": round(t_pre * 1e3, 3),
+                          "decode_tokens_per_s": round(batch * args.steps / dt, 1),
+                          "decode_ms_per_step": round(dt / args.steps * 1e3, 4),
+                          "decode_mean_context": round(mean_ctx, 1)}
+            drop(llm)
+        row["prefill_vs_qwen3"] = round(row["kugisun"]["prefill_tokens_per_s"]
+                                        / row["qwen3"]["prefill_tokens_per_s"], 3)
+        row["decode_vs_qwen3"] = round(row["kugisun"]["decode_tokens_per_s"]
+                                       / row["qwen3"]["decode_tokens_per_s"], 3)
+        if args.dtype == "bfloat16":
+            row["kernels_prefill"] = kugisun_kernels(sh, T, T, mfma_rate, read_bw)
+            row["kernels_decode"] = kugisun_kernels(sh, 1, prompt, mfma_rate, read_bw)
+        ops._workspaces.clear()
+        torch.cuda.empty_cache()
+        shapes[name] = row
+    first = shapes[names[0]]
+    print(json.dumps({
+        "metric": "kugisun_decode_tokens_per_s", "value": first["kugisun"]["decode_tokens_per_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["kugisun"]["decode_ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic", "config": {"model": f"Kugisun {names[0]} shape beside the dense Qwen3 "
+                                                 "decoder of equal size, random weights",
+                                        "batch": batch, "prompt_len": prompt, "prefill_tokens": T,
+                                        "parallelism": "single GPU"},
+        "measured_read_gbs": round(read_bw / 1e9, 1), "mfma_loop_tflops": round(mfma_rate / 1e12, 1),
+        "shapes": shapes}))
+    return 0
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel", "lodenex", "nupovik"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel", "lodenex", "nupovik",
+                             "kugisun"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="layer sizes (default: 8b for decode, 14b for continuous, 32b for "
                          "long-context)")
@@ -1330,6 +1642,8 @@ def main() -> int:
                     help="lodenex: only this shape (default: gqa, latent and mixed)")
     ap.add_argument("--nupovik-shape", default=None, choices=sorted(NUPOVIK_SHAPES),
                     help="nupovik: only this shape (default: all of them)")
+    ap.add_argument("--kugisun-shape", default=None, choices=sorted(KUGISUN_SHAPES),
+                    help="kugisun: only this shape (default: all of them)")
     ap.add_argument("--no-run-graphs", action="store_true",
                     help="decode steps in a row replay one graph per step instead of one for the run")
     args = ap.parse_args()
@@ -1339,7 +1653,8 @@ def main() -> int:
         return 2
     return {"decode": main_decode, "continuous": main_continuous,
             "long-context": main_long_context, "fezupel": main_fezupel,
-            "lodenex": main_lodenex, "nupovik": main_nupovik}[args.workload](args)
+            "lodenex": main_lodenex, "nupovik": main_nupovik,
+            "kugisun": main_kugisun}[args.workload](args)
 
 
 if __name__ == "__main__":

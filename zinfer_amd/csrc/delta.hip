@@ -28,76 +28,106 @@ __device__ __forceinline__ float dl_softplus(float z) {
 // out float32 [T, C].  Channels [0, unit_heads * hd) are heads of hd that leave as unit vectors
 // x / sqrt(sum x^2 + unit_eps), the first scaled_heads of them times `scale`.  State of a
 // request: [n - 1, C] floats at state + slot * state_stride + state_off, oldest row first.
-// update_state (only when every sequence of the step brings one token: a workgroup is then the
-// only reader of its state): the state is moved on by this kernel.
+// Grid (token, block of channels): the first head_blocks blocks hold hpb whole heads each, a
+// thread a channel (a head wider than the workgroup: one head a block, a thread several
+// channels), the others DL_CONV_THREADS plain channels.  A head's sum of squares is added up in
+// channel order by every thread of the head.
+// update_state (only when every sequence of the step brings one token: a thread is then the
+// only reader of its channel's kept rows): the state is moved on by this kernel.
+#define DL_CONV_THREADS 256
+#define DL_CONV_MAX_TAPS 8
+#define DL_CONV_PER_THREAD 4     // channels a thread takes of a head wider than the workgroup
+
 template <typename T>
-__global__ __launch_bounds__(256) void short_conv_kernel(
+__global__ __launch_bounds__(DL_CONV_THREADS) void short_conv_kernel(
     const T* __restrict__ src, long long src_stride, const float* __restrict__ taps, int n_taps,
     float* __restrict__ state, long long state_stride, long long state_off,
     const int* __restrict__ state_slots, const int* __restrict__ seq_index,
     const int* __restrict__ q_start, float* __restrict__ out, int C, int unit_heads, int hd,
-    int scaled_heads, float scale, float unit_eps, int update_state) {
+    int scaled_heads, float scale, float unit_eps, int update_state, int head_blocks, int hpb) {
 #pragma clang fp contract(off)
+  __shared__ float sq[DL_CONV_THREADS * DL_CONV_PER_THREAD];
   const int t = blockIdx.x;
   const int s = seq_index[t];
   const int i0 = t - q_start[s];                       // the token's place in its portion
   float* st = state + (size_t)state_slots[s] * state_stride + state_off;
   const int hist = n_taps - 1;
   auto conv = [&](int c) -> float {
+    float x[DL_CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < DL_CONV_MAX_TAPS; ++j) {
+      x[j] = 0.f;
+      if (j < n_taps) {
+        const int back = hist - j;                     // rows before the token's own
+        if (back <= i0) x[j] = load_as_float<T>(src + (size_t)(t - back) * src_stride + c);
+        else x[j] = st[(size_t)(hist + i0 - back) * C + c];
+      }
+    }
     float acc = 0.f;
-    for (int j = 0; j < n_taps; ++j) {
-      const int back = hist - j;                       // rows before the token's own
-      float x;
-      if (back <= i0) x = load_as_float<T>(src + (size_t)(t - back) * src_stride + c);
-      else x = st[(size_t)(hist + i0 - back) * C + c];
-      acc = acc + taps[(size_t)c * n_taps + j] * x;
+#pragma unroll
+    for (int j = 0; j < DL_CONV_MAX_TAPS; ++j)
+      if (j < n_taps) acc = acc + taps[(size_t)c * n_taps + j] * x[j];
+    if (update_state) {
+      // the kept rows move on by one: rows 1 .. of what was read, then the token's own
+#pragma unroll
+      for (int j = 1; j < DL_CONV_MAX_TAPS; ++j)
+        if (j < n_taps) st[(size_t)(j - 1) * C + c] = x[j];
     }
     return dl_silu(acc);
   };
-  const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
   float* o = out + (size_t)t * C;
-  for (int head = wave; head < unit_heads; head += blockDim.x / ZF_WAVE) {
-    float ss = 0.f;
-    for (int d = lane; d < hd; d += ZF_WAVE) {
-      const float v = conv(head * hd + d);
-      o[head * hd + d] = v;
-      ss += v * v;
-    }
-    ss = wave_sum(ss);
-    float inv = 1.0f / sqrtf(ss + unit_eps);
-    if (head < scaled_heads) inv = inv * scale;
-    // (a lane reads back what it wrote itself)
-    for (int d = lane; d < hd; d += ZF_WAVE) o[head * hd + d] = o[head * hd + d] * inv;
+  const int b = blockIdx.y;
+  if (b >= head_blocks) {
+    const int c = unit_heads * hd + (b - head_blocks) * DL_CONV_THREADS + threadIdx.x;
+    if (c < C) o[c] = conv(c);
+    return;
   }
-  for (int c = unit_heads * hd + threadIdx.x; c < C; c += blockDim.x) o[c] = conv(c);
-  if (update_state) {
-    __syncthreads();                                   // every channel's old rows have been read
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-      for (int r = 0; r + 1 < hist; ++r) st[(size_t)r * C + c] = st[(size_t)(r + 1) * C + c];
-      if (hist > 0) st[(size_t)(hist - 1) * C + c] = load_as_float<T>(src + (size_t)t * src_stride + c);
-    }
+  const int per = hpb > 0 ? 1 : (hd + DL_CONV_THREADS - 1) / DL_CONV_THREADS;
+  const int head = hpb > 0 ? b * hpb + threadIdx.x / hd : b;
+  const int d0 = hpb > 0 ? threadIdx.x % hd : threadIdx.x;
+  const bool mine = hpb > 0 ? (threadIdx.x < hpb * hd && head < unit_heads) : true;
+  float v[DL_CONV_PER_THREAD];
+#pragma unroll
+  for (int j = 0; j < DL_CONV_PER_THREAD; ++j) {
+    v[j] = 0.f;
+    const int dd = d0 + j * DL_CONV_THREADS;
+    if (j < per && mine && dd < hd) v[j] = conv(head * hd + dd);
+    if (j < per) sq[threadIdx.x + j * DL_CONV_THREADS] = v[j] * v[j];
+  }
+  __syncthreads();
+  if (!mine) return;
+  // the head's squares in channel order: every thread of the head adds the same numbers
+  const float* hs = hpb > 0 ? sq + (threadIdx.x / hd) * hd : sq;
+  float ss = 0.f;
+  for (int i = 0; i < hd; ++i) ss += hs[i];
+  float inv = 1.0f / sqrtf(ss + unit_eps);
+  if (head < scaled_heads) inv = inv * scale;
+#pragma unroll
+  for (int j = 0; j < DL_CONV_PER_THREAD; ++j) {
+    const int dd = d0 + j * DL_CONV_THREADS;
+    if (j < per && dd < hd) o[head * hd + dd] = v[j] * inv;
   }
 }
 
-// The state after a step: the last n - 1 rows the convolution has seen.  A workgroup a sequence.
+// The state after a step: the last n - 1 rows the convolution has seen.  Grid (sequence, block of
+// channels), a thread a channel.
 template <typename T>
-__global__ __launch_bounds__(256) void short_conv_state_kernel(
+__global__ __launch_bounds__(DL_CONV_THREADS) void short_conv_state_kernel(
     const T* __restrict__ src, long long src_stride, int n_taps, float* __restrict__ state,
     long long state_stride, long long state_off, const int* __restrict__ state_slots,
     const int* __restrict__ q_start, int C) {
   const int s = blockIdx.x;
   const int first = q_start[s], len = q_start[s + 1] - first;
-  if (len <= 0) return;
+  const int c = blockIdx.y * DL_CONV_THREADS + threadIdx.x;
+  if (len <= 0 || c >= C) return;
   float* st = state + (size_t)state_slots[s] * state_stride + state_off;
   const int hist = n_taps - 1;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    // row r of the new state is the portion's row len - hist + r, or (before the portion) the
-    // old state's row r + len, which lies behind the row being written: ascending r is safe
-    for (int r = 0; r < hist; ++r) {
-      const int i = len - hist + r;
-      st[(size_t)r * C + c] = i >= 0 ? load_as_float<T>(src + (size_t)(first + i) * src_stride + c)
-                                     : st[(size_t)(r + len) * C + c];
-    }
+  // row r of the new state is the portion's row len - hist + r, or (before the portion) the
+  // old state's row r + len, which lies behind the row being written: ascending r is safe
+  for (int r = 0; r < hist; ++r) {
+    const int i = len - hist + r;
+    st[(size_t)r * C + c] = i >= 0 ? load_as_float<T>(src + (size_t)(first + i) * src_stride + c)
+                                   : st[(size_t)(r + len) * C + c];
   }
 }
 
@@ -108,16 +138,23 @@ extern "C" int zf_short_conv(const void* src, int dtype, long long src_stride, c
                              int unit_heads, int hd, int scaled_heads, float scale,
                              float unit_eps, int single_tokens, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (C <= 0 || n_taps < 1 || unit_heads < 0 || hd < 1 || (size_t)unit_heads * hd > (size_t)C ||
-      scaled_heads > unit_heads || n_seqs < 1 || (single_tokens && T != n_seqs))
+  if (C <= 0 || n_taps < 1 || n_taps > DL_CONV_MAX_TAPS || unit_heads < 0 || hd < 1 ||
+      (size_t)unit_heads * hd > (size_t)C || scaled_heads > unit_heads || n_seqs < 1 ||
+      (single_tokens && T != n_seqs) || hd > DL_CONV_THREADS * DL_CONV_PER_THREAD)
     return -2;
+  // whole heads a block where a head fits a workgroup, else one head a block
+  const int hpb = hd <= DL_CONV_THREADS ? DL_CONV_THREADS / hd : 0;
+  const int head_blocks = unit_heads == 0 ? 0 : (hpb > 0 ? (unit_heads + hpb - 1) / hpb : unit_heads);
+  const int plain = C - unit_heads * hd;
+  const dim3 grid(T, head_blocks + (plain + DL_CONV_THREADS - 1) / DL_CONV_THREADS);
+  const dim3 sgrid(n_seqs, (C + DL_CONV_THREADS - 1) / DL_CONV_THREADS);
 #define DL_CONV_LAUNCH(TT)                                                                        \
-  hipLaunchKernelGGL(short_conv_kernel<TT>, dim3(T), dim3(256), 0, stream, (const TT*)src,       \
-                     src_stride, taps, n_taps, state, state_stride, state_off, state_slots,      \
-                     seq_index, q_start, out, C, unit_heads, hd, scaled_heads, scale, unit_eps,  \
-                     single_tokens);                                                              \
+  hipLaunchKernelGGL(short_conv_kernel<TT>, grid, dim3(DL_CONV_THREADS), 0, stream,              \
+                     (const TT*)src, src_stride, taps, n_taps, state, state_stride, state_off,   \
+                     state_slots, seq_index, q_start, out, C, unit_heads, hd, scaled_heads,      \
+                     scale, unit_eps, single_tokens, head_blocks, hpb);                          \
   if (!single_tokens && n_taps > 1)                                                               \
-    hipLaunchKernelGGL(short_conv_state_kernel<TT>, dim3(n_seqs), dim3(256), 0, stream,          \
+    hipLaunchKernelGGL(short_conv_state_kernel<TT>, sgrid, dim3(DL_CONV_THREADS), 0, stream,     \
                        (const TT*)src, src_stride, n_taps, state, state_stride, state_off,       \
                        state_slots, q_start, C)
   if (dtype == ZF_F32) { DL_CONV_LAUNCH(float); } else { DL_CONV_LAUNCH(bf16_t); }
@@ -127,13 +164,32 @@ extern "C" int zf_short_conv(const void* src, int dtype, long long src_stride, c
 // ------------------------------------------------------------------ the recurrence
 #define DL_STAGE 16            // tokens staged in LDS at a time
 #define DL_MAX_LANES 16        // lanes that share a column's key channels
+#define DL_PF 4                // 16-byte pieces of q and of k, and values of v, a thread fetches ahead
+
+// The sum over the CG lanes (a power of two up to 16, aligned in a row of 16 lanes) that share a
+// column, in every one of them, through the data-parallel lane moves: neighbours, pairs, then the
+// mirrored half row and row (a lane and its mirror hold sums over different halves).
+template <int CTRL>
+__device__ __forceinline__ float dl_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dl_lanes_sum(float v, int CG) {
+  if (CG >= 2) v += dl_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  if (CG >= 4) v += dl_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if (CG >= 8) v += dl_move<0x141>(v);     // row_half_mirror
+  if (CG >= 16) v += dl_move<0x140>(v);    // row_mirror
+  return v;
+}
 
 // A thread holds R key channels of one value column of S; CG lanes side by side hold the
 // column's P = CG * R channels (zeros beyond d).  A request's matrices lie [head][column][P] in
 // its state, so a thread's channels are consecutive.  Grid (column tiles, heads, sequences).
 // qkv float32 [T, C]: q heads at q_off, k heads at k_off (KH heads of d each), v heads at v_off
 // (H heads of dv); ab float32 [T, 2 H]: the decays' numbers z_a, then the step sizes' z_b.
-template <int R>
+// Sixteen tokens at a time lie in LDS; the next sixteen are asked for before these are walked
+// (16-byte pieces, where the rows' offsets allow: VEC), and a token's operands are read from LDS
+// while the token before it is computed.
+template <int R, bool VEC>
 __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ qkv, int C, int q_off, int k_off, int v_off,
     const float* __restrict__ ab, const float* __restrict__ a_log,
@@ -156,7 +212,7 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   const int tid = threadIdx.x, nthreads = blockDim.x;
   const int cg = tid % CG, col_l = tid / CG;
   const int col = blockIdx.x * cols + col_l;
-  const bool live = col_l < cols && col < dv;
+  const bool live = col < dv;
   float* S_mem = state + (size_t)state_slots[seq] * state_stride
                  + ((size_t)h * dv + (live ? col : 0)) * P + cg * R;
   float S[R];
@@ -168,25 +224,85 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   const float decay_rate = expf(a_log[h]);
   const float dtb = dt_bias[h];
   const int wave = tid / ZF_WAVE, lane = tid % ZF_WAVE, nwaves = (nthreads + ZF_WAVE - 1) / ZF_WAVE;
+  const int P4 = P / 4;
+  // what a thread fetches ahead: pieces tid, tid + nthreads, ... of the stage's q and k rows,
+  // one value of its v columns, and (the first threads) a token's two numbers
+  float4 fq[DL_PF], fk[DL_PF];
+  float fv[DL_PF], fa = 0.f, fb = 0.f;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  auto fetch = [&](int t0, int n) {
+    if constexpr (VEC) {
+#pragma unroll
+      for (int j = 0; j < DL_PF; ++j) {
+        const int i = tid + j * nthreads;
+        fq[j] = fk[j] = zero4;
+        if (i < n * P4) {
+          const int tok = i / P4, c = (i % P4) * 4;
+          const float* row = qkv + (size_t)(first + t0 + tok) * C;
+          if (c < d) {
+            fq[j] = *(const float4*)(row + q_off + kh * d + c);
+            fk[j] = *(const float4*)(row + k_off + kh * d + c);
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < DL_PF; ++j) {
+        const int i = tid + j * nthreads;
+        fv[j] = 0.f;
+        if (i < n * cols) {
+          const int tok = i / cols, c = blockIdx.x * cols + i % cols;
+          if (c < dv) fv[j] = qkv[(size_t)(first + t0 + tok) * C + v_off + h * dv + c];
+        }
+      }
+      if (tid < n) {
+        const float* z = ab + (size_t)(first + t0 + tid) * 2 * H;
+        fa = z[h];
+        fb = z[H + h];
+      }
+    }
+  };
+  auto stage = [&](int t0, int n) {
+    if constexpr (VEC) {
+#pragma unroll
+      for (int j = 0; j < DL_PF; ++j) {
+        const int i = tid + j * nthreads;
+        if (i < n * P4) {
+          *(float4*)(qs + 4 * i) = fq[j];
+          *(float4*)(ks + 4 * i) = fk[j];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < DL_PF; ++j)
+        if (tid + j * nthreads < n * cols) vs[tid + j * nthreads] = fv[j];
+      if (tid < n) {
+        gs[tid] = expf(-(decay_rate * dl_softplus(fa + dtb)));
+        bs[tid] = 1.0f / (1.0f + expf(-fb));
+      }
+    } else {
+      for (int i = tid; i < n * P; i += nthreads) {
+        const int tok = i / P, c = i % P;
+        const float* row = qkv + (size_t)(first + t0 + tok) * C;
+        qs[i] = c < d ? row[q_off + kh * d + c] : 0.f;
+        ks[i] = c < d ? row[k_off + kh * d + c] : 0.f;
+      }
+      for (int i = tid; i < n * cols; i += nthreads) {
+        const int tok = i / cols, c = blockIdx.x * cols + i % cols;
+        vs[i] = c < dv ? qkv[(size_t)(first + t0 + tok) * C + v_off + h * dv + c] : 0.f;
+      }
+      if (tid < n) {
+        const float* z = ab + (size_t)(first + t0 + tid) * 2 * H;
+        gs[tid] = expf(-(decay_rate * dl_softplus(z[h] + dtb)));
+        bs[tid] = 1.0f / (1.0f + expf(-z[H + h]));
+      }
+    }
+  };
+  fetch(0, min(DL_STAGE, len));
   for (int t0 = 0; t0 < len; t0 += DL_STAGE) {
     const int n = min(DL_STAGE, len - t0);
     __syncthreads();                        // the tokens staged before are done with
-    for (int i = tid; i < n * P; i += nthreads) {
-      const int tok = i / P, c = i % P;
-      const float* row = qkv + (size_t)(first + t0 + tok) * C;
-      qs[i] = c < d ? row[q_off + kh * d + c] : 0.f;
-      ks[i] = c < d ? row[k_off + kh * d + c] : 0.f;
-    }
-    for (int i = tid; i < n * cols; i += nthreads) {
-      const int tok = i / cols, c = blockIdx.x * cols + i % cols;
-      vs[i] = c < dv ? qkv[(size_t)(first + t0 + tok) * C + v_off + h * dv + c] : 0.f;
-    }
-    if (tid < n) {
-      const float* z = ab + (size_t)(first + t0 + tid) * 2 * H;
-      gs[tid] = expf(-(decay_rate * dl_softplus(z[h] + dtb)));
-      bs[tid] = 1.0f / (1.0f + expf(-z[H + h]));
-    }
+    stage(t0, n);
     __syncthreads();
+    if (t0 + DL_STAGE < len) fetch(t0 + DL_STAGE, min(DL_STAGE, len - t0 - DL_STAGE));
     for (int tok = wave; tok < n; tok += nwaves) {
       float dot = 0.f;
       for (int c = lane; c < P; c += ZF_WAVE) dot += qs[tok * P + c] * ks[tok * P + c];
@@ -194,30 +310,38 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
       if (lane == 0) ds[tok] = dot;
     }
     __syncthreads();
-    for (int tok = 0; tok < n; ++tok) {
+    // a token's operands are read a token ahead
+    float kk[R], qq[R], g, b, v, qk;
+    auto read = [&](int tok) {
       const float* qrow = qs + tok * P + cg * R;
       const float* krow = ks + tok * P + cg * R;
-      float kk[R];
-      float r0 = 0.f, r1 = 0.f, p0 = 0.f, p1 = 0.f;
 #pragma unroll
       for (int r = 0; r < R; r += 4) {
         const float4 kv = *(const float4*)(krow + r);
         const float4 qv = *(const float4*)(qrow + r);
         kk[r] = kv.x; kk[r + 1] = kv.y; kk[r + 2] = kv.z; kk[r + 3] = kv.w;
-        r0 += kv.x * S[r]; r1 += kv.y * S[r + 1]; r0 += kv.z * S[r + 2]; r1 += kv.w * S[r + 3];
-        p0 += qv.x * S[r]; p1 += qv.y * S[r + 1]; p0 += qv.z * S[r + 2]; p1 += qv.w * S[r + 3];
+        qq[r] = qv.x; qq[r + 1] = qv.y; qq[r + 2] = qv.z; qq[r + 3] = qv.w;
       }
-      float rs = r0 + r1, ps = p0 + p1;
-      for (int off = 1; off < CG; off <<= 1) {
-        rs += __shfl_xor(rs, off, ZF_WAVE);
-        ps += __shfl_xor(ps, off, ZF_WAVE);
-      }
-      const float g = gs[tok];
-      const float w = bs[tok] * (vs[tok * cols + (col_l < cols ? col_l : 0)] - g * rs);
+      g = gs[tok]; b = bs[tok]; v = vs[tok * cols + col_l]; qk = ds[tok];
+    };
+    read(0);
+    for (int tok = 0; tok < n; ++tok) {
+      float r0 = 0.f, r1 = 0.f, p0 = 0.f, p1 = 0.f;
+      float kc[R];
 #pragma unroll
-      for (int r = 0; r < R; ++r) S[r] = g * S[r] + kk[r] * w;
+      for (int r = 0; r < R; r += 2) {
+        kc[r] = kk[r]; kc[r + 1] = kk[r + 1];
+        r0 += kk[r] * S[r]; r1 += kk[r + 1] * S[r + 1];
+        p0 += qq[r] * S[r]; p1 += qq[r + 1] * S[r + 1];
+      }
+      const float gc = g, bc = b, vc = v, qkc = qk;
+      if (tok + 1 < n) read(tok + 1);
+      const float rs = dl_lanes_sum(r0 + r1, CG), ps = dl_lanes_sum(p0 + p1, CG);
+      const float w = bc * (vc - gc * rs);
+#pragma unroll
+      for (int r = 0; r < R; ++r) S[r] = gc * S[r] + kc[r] * w;
       if (live && cg == 0)
-        out[(size_t)(first + t0 + tok) * H * dv + (size_t)h * dv + col] = g * ps + ds[tok] * w;
+        out[(size_t)(first + t0 + tok) * H * dv + (size_t)h * dv + col] = gc * ps + qkc * w;
     }
   }
   if (live) {
@@ -242,16 +366,24 @@ extern "C" int zf_delta_recurrence(const float* qkv, int C, int q_off, int k_off
     return -2;
   const dim3 grid((dv + cols - 1) / cols, H, n_seqs), block(threads);
   const size_t smem = (size_t)(DL_STAGE * (2 * R * CG + cols) + 3 * DL_STAGE) * sizeof(float);
+  // 16-byte pieces: every row offset a multiple of four floats, and few enough pieces a thread
+  const bool vec = C % 4 == 0 && q_off % 4 == 0 && k_off % 4 == 0 && d % 4 == 0 &&
+                   ((uintptr_t)qkv % 16) == 0 &&
+                   DL_STAGE * (R * CG / 4) <= DL_PF * threads && DL_STAGE * cols <= DL_PF * threads &&
+                   DL_STAGE <= threads;
 #define DL_REC_LAUNCH(RR)                                                                        \
-  hipLaunchKernelGGL(delta_recurrence_kernel<RR>, grid, block, smem, stream, qkv, C, q_off,      \
-                     k_off, v_off, ab, a_log, dt_bias, state, state_stride, state_slots,         \
-                     q_start, out, H, KH, d, dv, CG, cols)
+  if (vec)                                                                                       \
+    hipLaunchKernelGGL((delta_recurrence_kernel<RR, true>), grid, block, smem, stream, qkv, C,   \
+                       q_off, k_off, v_off, ab, a_log, dt_bias, state, state_stride,             \
+                       state_slots, q_start, out, H, KH, d, dv, CG, cols);                       \
+  else                                                                                           \
+    hipLaunchKernelGGL((delta_recurrence_kernel<RR, false>), grid, block, smem, stream, qkv, C,  \
+                       q_off, k_off, v_off, ab, a_log, dt_bias, state, state_stride,             \
+                       state_slots, q_start, out, H, KH, d, dv, CG, cols)
   switch (R) {
     case 8: DL_REC_LAUNCH(8); break;
     case 12: DL_REC_LAUNCH(12); break;
     case 16: DL_REC_LAUNCH(16); break;
-    case 24: DL_REC_LAUNCH(24); break;
-    case 32: DL_REC_LAUNCH(32); break;
     default: return -2;
   }
   ZF_CHECK_LAUNCH();

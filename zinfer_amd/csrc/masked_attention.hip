@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
   const float pos = (float)positions[t];
   const float* have = nullptr;          // the frequencies the tables in LDS were made from
   float have_mag = 0.f;
-  for (int si = 0; si < segs.n; ++si) {
+  for (int si = blockIdx.y; si < segs.n; si += gridDim.y) {
     const RowSegment& g = segs.s[si];
     const T* x = row + g.src_off;
     float inv = 1.f;
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void project_rows_vec8_kernel(
   const float pos = (float)positions[t];
   const float* have = nullptr;
   float have_mag = 0.f;
-  for (int si = 0; si < segs.n; ++si) {
+  for (int si = blockIdx.y; si < segs.n; si += gridDim.y) {
     const RowSegment& g = segs.s[si];
     const bf16_t* x = row + g.src_off;
     const int n8 = g.width / 8;
@@ -349,15 +349,15 @@ extern "C" int zf_project_rows(const void* src, int dtype, long long src_stride,
         && (g.to_pool || g.dst_stride % 8 == 0) && (g.gain == nullptr || (uintptr_t)g.gain % 16 == 0);
   }
   if (vec8) {
-    hipLaunchKernelGGL(project_rows_vec8_kernel, dim3(T), dim3(256), 0, stream,
+    hipLaunchKernelGGL(project_rows_vec8_kernel, dim3(T, n_segs), dim3(256), 0, stream,
                        (const bf16_t*)src, src_stride, positions, slot_mapping, page_size, segs);
     ZF_CHECK_LAUNCH();
   }
   if (dtype == ZF_F32)
-    hipLaunchKernelGGL(project_rows_kernel<float>, dim3(T), dim3(256), 0, stream,
+    hipLaunchKernelGGL(project_rows_kernel<float>, dim3(T, n_segs), dim3(256), 0, stream,
                        (const float*)src, src_stride, positions, slot_mapping, page_size, segs);
   else
-    hipLaunchKernelGGL(project_rows_kernel<bf16_t>, dim3(T), dim3(256), 0, stream,
+    hipLaunchKernelGGL(project_rows_kernel<bf16_t>, dim3(T, n_segs), dim3(256), 0, stream,
                        (const bf16_t*)src, src_stride, positions, slot_mapping, page_size, segs);
   ZF_CHECK_LAUNCH();
 }

@@ -336,7 +336,8 @@ extern "C" int zf_embed_position(const void* table, const void* pos_table, int t
 // of the copies at the end, both between two sublayers.  The sums run over s in ascending order.
 #define STREAMS_MAX 8
 
-template <typename TO>
+// V: columns a thread takes side by side (4: 16-byte loads and stores; W a multiple of 4)
+template <typename TO, int V>
 __global__ __launch_bounds__(256) void streams_step_kernel(
     float* __restrict__ x, long long copy_stride, int S, const float* __restrict__ y0,
     const float* __restrict__ y1, float c0, float c1, const float* __restrict__ M,
@@ -345,42 +346,76 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
 #pragma clang fp contract(off)
   extern __shared__ float u_row[];
   __shared__ float red[16];
+  __shared__ float cm[STREAMS_MAX * STREAMS_MAX], cb[STREAMS_MAX], ca[STREAMS_MAX];
+  // the coefficients once a workgroup
+  if (threadIdx.x < S * S && M != nullptr) cm[threadIdx.x] = M[threadIdx.x];
+  if (threadIdx.x < S) {
+    if (b != nullptr) cb[threadIdx.x] = b[threadIdx.x];
+    ca[threadIdx.x] = a != nullptr ? a[threadIdx.x] : 1.0f;
+  }
+  __syncthreads();
   const size_t row = (size_t)blockIdx.x * W;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float v[STREAMS_MAX];
+  for (int i = threadIdx.x * V; i < W; i += blockDim.x * V) {
+    float v[STREAMS_MAX][V];
 #pragma unroll
-    for (int s = 0; s < STREAMS_MAX; ++s) v[s] = s < S ? x[s * copy_stride + row + i] : 0.f;
+    for (int s = 0; s < STREAMS_MAX; ++s) {
+      if (s < S) {
+        if constexpr (V == 4) {
+          const float4 q = *(const float4*)(x + s * copy_stride + row + i);
+          v[s][0] = q.x; v[s][1] = q.y; v[s][2] = q.z; v[s][3] = q.w;
+        } else {
+          v[s][0] = x[s * copy_stride + row + i];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[s][e] = 0.f;
+      }
+    }
     if (y0 != nullptr) {
-      float y = c0 * y0[row + i];
-      if (y1 != nullptr) y = y + c1 * y1[row + i];
-      float n[STREAMS_MAX];
+      float y[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        y[e] = c0 * y0[row + i + e];
+        if (y1 != nullptr) y[e] = y[e] + c1 * y1[row + i + e];
+      }
+      float n[STREAMS_MAX][V];
 #pragma unroll
       for (int t = 0; t < STREAMS_MAX; ++t) {
         if (t >= S) continue;
-        float acc = 0.f;
 #pragma unroll
-        for (int s = 0; s < STREAMS_MAX; ++s)
-          if (s < S) acc = acc + M[s * S + t] * v[s];
-        n[t] = acc + b[t] * y;
+        for (int e = 0; e < V; ++e) {
+          float acc = 0.f;
+#pragma unroll
+          for (int s = 0; s < STREAMS_MAX; ++s)
+            if (s < S) acc = acc + cm[s * S + t] * v[s][e];
+          n[t][e] = acc + cb[t] * y[e];
+        }
       }
 #pragma unroll
       for (int t = 0; t < STREAMS_MAX; ++t)
         if (t < S) {
-          v[t] = n[t];
-          x[t * copy_stride + row + i] = n[t];
+#pragma unroll
+          for (int e = 0; e < V; ++e) v[t][e] = n[t][e];
+          if constexpr (V == 4)
+            *(float4*)(x + t * copy_stride + row + i) = make_float4(n[t][0], n[t][1], n[t][2], n[t][3]);
+          else
+            x[t * copy_stride + row + i] = n[t][0];
         }
     }
     if (do_read) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < STREAMS_MAX; ++s)
-        if (s < S) u = u + (a != nullptr ? a[s] : 1.0f) * v[s];
-      if (gain == nullptr) {
-        store_from_float<TO>(out + row + i, u);
-      } else {
-        u_row[i] = u;
-        ss += u * u;
+      for (int e = 0; e < V; ++e) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; ++s)
+          if (s < S) u = u + ca[s] * v[s][e];
+        if (gain == nullptr) {
+          store_from_float<TO>(out + row + i + e, u);
+        } else {
+          u_row[i + e] = u;
+          ss += u * u;
+        }
       }
     }
   }
@@ -388,8 +423,11 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)W + eps);
   // (a thread reads back the columns it wrote itself)
-  for (int i = threadIdx.x; i < W; i += blockDim.x)
-    store_from_float<TO>(out + row + i, u_row[i] * inv * gain[i]);
+  for (int i = threadIdx.x * V; i < W; i += blockDim.x * V) {
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+      store_from_float<TO>(out + row + i + e, u_row[i + e] * inv * gain[i + e]);
+  }
 }
 
 // x [S, T, W] (copy_stride elements from one copy to the next).  y0 null: no write; else y1
@@ -406,12 +444,15 @@ extern "C" int zf_streams_step(float* x, long long copy_stride, int S, const flo
       (do_read && gain == nullptr && out_dtype != ZF_F32))
     return -2;
   const size_t smem = (size_t)W * sizeof(float);
-  if (out_dtype == ZF_F32)
-    hipLaunchKernelGGL(streams_step_kernel<float>, dim3(T), dim3(256), smem, stream, x,
-                       copy_stride, S, y0, y1, c0, c1, M, b, a, gain, eps, (float*)out, W, do_read);
-  else
-    hipLaunchKernelGGL(streams_step_kernel<bf16_t>, dim3(T), dim3(256), smem, stream, x,
-                       copy_stride, S, y0, y1, c0, c1, M, b, a, gain, eps, (bf16_t*)out, W,
-                       do_read);
+  const bool vec = W % 4 == 0 && copy_stride % 4 == 0 && ((uintptr_t)x % 16) == 0 &&
+                   (y0 == nullptr || (uintptr_t)y0 % 16 == 0);
+#define STREAMS_LAUNCH(TT, VV)                                                                   \
+  hipLaunchKernelGGL((streams_step_kernel<TT, VV>), dim3(T), dim3(256), smem, stream, x,         \
+                     copy_stride, S, y0, y1, c0, c1, M, b, a, gain, eps, (TT*)out, W, do_read)
+  if (out_dtype == ZF_F32) {
+    if (vec) STREAMS_LAUNCH(float, 4); else STREAMS_LAUNCH(float, 1);
+  } else {
+    if (vec) STREAMS_LAUNCH(bf16_t, 4); else STREAMS_LAUNCH(bf16_t, 1);
+  }
   ZF_CHECK_LAUNCH();
 }

@@ -2616,6 +2616,8 @@ def streams_step(x: torch.Tensor, branches=(), mix: Optional[torch.Tensor] = Non
 DELTA_MAX_KEY_DIM = 256
 DELTA_CHANNELS = (8, 12, 16)      # key channels a thread holds (instantiations in delta.hip)
 DELTA_MAX_LANES = 16              # lanes that share a column's key channels
+SHORT_CONV_MAX_TAPS = 8           # DL_CONV_MAX_TAPS in delta.hip
+SHORT_CONV_MAX_HEAD_DIM = 1024    # a head that leaves as a unit vector lies in one workgroup
 
 
 def delta_plan(key_dim: int) -> Tuple[int, int]:
@@ -2679,6 +2681,7 @@ def short_conv(src: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, state
             or state_offset < 0 or state_offset + (n - 1) * C > state.shape[1] \
             or seq_index.shape[0] != T or q_start.shape[0] != n_seqs + 1 \
             or unit_heads < 0 or head_dim < 1 or unit_heads * head_dim > C \
+            or n > SHORT_CONV_MAX_TAPS or head_dim > SHORT_CONV_MAX_HEAD_DIM \
             or scaled_heads > unit_heads or (single_tokens and T != n_seqs):
         raise KernelUnavailable(f"short_conv: src {tuple(src.shape)}, taps {tuple(taps.shape)} "
                                 f"{taps.dtype}, out {tuple(out.shape)} {out.dtype}, state "

@@ -33,6 +33,9 @@ class GatedDeltaRule(Mixer):
         if s.head_dim > ops.DELTA_MAX_KEY_DIM:
             raise ConfigError(f"InvalidHeadDim: dim={s.head_dim}: the delta rule's kernel takes "
                               f"key sizes up to {ops.DELTA_MAX_KEY_DIM}")
+        if s.conv_taps > ops.SHORT_CONV_MAX_TAPS:
+            raise ConfigError(f"conv={s.conv_taps}: the convolution kernel takes up to "
+                              f"{ops.SHORT_CONV_MAX_TAPS} taps")
         self.qk_width = s.n_kv_heads * s.head_dim
         self.v_width = s.n_heads * s.value_dim
         self.conv_width = 2 * self.qk_width + self.v_width
