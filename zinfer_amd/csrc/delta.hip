@@ -23,15 +23,33 @@ __device__ __forceinline__ float dl_softplus(float z) {
   return z > 20.f ? z : log1pf(expf(z));
 }
 
+// The sum over the CG lanes (a power of two up to 16, aligned in a row of 16 lanes) that share a
+// column, in every one of them, through the data-parallel lane moves: neighbours, pairs, then the
+// mirrored half row and row (a lane and its mirror hold sums over different halves).
+template <int CTRL>
+__device__ __forceinline__ float dl_move(float v) {
+  // (every lane has a source lane: the value a lane without one would keep is never used)
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL,
+                                                    0xf, 0xf, true));
+}
+template <int CG>
+__device__ __forceinline__ float dl_lanes_sum(float v) {
+  if constexpr (CG >= 2) v += dl_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  if constexpr (CG >= 4) v += dl_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if constexpr (CG >= 8) v += dl_move<0x141>(v);     // row_half_mirror
+  if constexpr (CG >= 16) v += dl_move<0x140>(v);    // row_mirror
+  return v;
+}
+
 // ------------------------------------------------------------------ short convolutions
 // src [T, >= C] (row stride given), taps [C, n] float32 (the last column is the token's own),
 // out float32 [T, C].  Channels [0, unit_heads * hd) are heads of hd that leave as unit vectors
 // x / sqrt(sum x^2 + unit_eps), the first scaled_heads of them times `scale`.  State of a
 // request: [n - 1, C] floats at state + slot * state_stride + state_off, oldest row first.
 // Grid (token, block of channels): the first head_blocks blocks hold hpb whole heads each, a
-// thread a channel (a head wider than the workgroup: one head a block, a thread several
-// channels), the others DL_CONV_THREADS plain channels.  A head's sum of squares is added up in
-// channel order by every thread of the head.
+// head in one, two or four whole waves and a thread a channel (a head wider than the workgroup:
+// a thread several channels), the others DL_CONV_THREADS plain channels.  A head's sum of
+// squares is added up over a wave's lanes and then over the head's waves in their order.
 // update_state (only when every sequence of the step brings one token: a thread is then the
 // only reader of its channel's kept rows): the state is moved on by this kernel.
 #define DL_CONV_THREADS 256
@@ -46,7 +64,7 @@ __global__ __launch_bounds__(DL_CONV_THREADS) void short_conv_kernel(
     const int* __restrict__ q_start, float* __restrict__ out, int C, int unit_heads, int hd,
     int scaled_heads, float scale, float unit_eps, int update_state, int head_blocks, int hpb) {
 #pragma clang fp contract(off)
-  __shared__ float sq[DL_CONV_THREADS * DL_CONV_PER_THREAD];
+  __shared__ float sq[DL_CONV_THREADS / ZF_WAVE];
   const int t = blockIdx.x;
   const int s = seq_index[t];
   const int i0 = t - q_start[s];                       // the token's place in its portion
@@ -82,29 +100,36 @@ __global__ __launch_bounds__(DL_CONV_THREADS) void short_conv_kernel(
     if (c < C) o[c] = conv(c);
     return;
   }
-  const int per = hpb > 0 ? 1 : (hd + DL_CONV_THREADS - 1) / DL_CONV_THREADS;
-  const int head = hpb > 0 ? b * hpb + threadIdx.x / hd : b;
-  const int d0 = hpb > 0 ? threadIdx.x % hd : threadIdx.x;
-  const bool mine = hpb > 0 ? (threadIdx.x < hpb * hd && head < unit_heads) : true;
+  // a head takes tph threads, whole waves of them (hpb heads a block), a thread `per` channels
+  const int tph = DL_CONV_THREADS / hpb;
+  const int per = (hd + tph - 1) / tph;
+  const int head = b * hpb + threadIdx.x / tph;
+  const int d0 = threadIdx.x % tph;
+  const bool mine = head < unit_heads;
   float v[DL_CONV_PER_THREAD];
+  float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < DL_CONV_PER_THREAD; ++j) {
     v[j] = 0.f;
-    const int dd = d0 + j * DL_CONV_THREADS;
+    const int dd = d0 + j * tph;
     if (j < per && mine && dd < hd) v[j] = conv(head * hd + dd);
-    if (j < per) sq[threadIdx.x + j * DL_CONV_THREADS] = v[j] * v[j];
+    ss += v[j] * v[j];
   }
+  // over the lanes of a wave, then over the head's waves in their order
+  ss = dl_lanes_sum<16>(ss);
+  ss += __shfl_xor(ss, 16, ZF_WAVE);
+  ss += __shfl_xor(ss, 32, ZF_WAVE);
+  const int wave = threadIdx.x / ZF_WAVE, wph = tph / ZF_WAVE;
+  if (threadIdx.x % ZF_WAVE == 0) sq[wave] = ss;
   __syncthreads();
   if (!mine) return;
-  // the head's squares in channel order: every thread of the head adds the same numbers
-  const float* hs = hpb > 0 ? sq + (threadIdx.x / hd) * hd : sq;
-  float ss = 0.f;
-  for (int i = 0; i < hd; ++i) ss += hs[i];
-  float inv = 1.0f / sqrtf(ss + unit_eps);
+  float total = 0.f;
+  for (int w = 0; w < wph; ++w) total += sq[(wave / wph) * wph + w];
+  float inv = 1.0f / sqrtf(total + unit_eps);
   if (head < scaled_heads) inv = inv * scale;
 #pragma unroll
   for (int j = 0; j < DL_CONV_PER_THREAD; ++j) {
-    const int dd = d0 + j * DL_CONV_THREADS;
+    const int dd = d0 + j * tph;
     if (j < per && dd < hd) o[head * hd + dd] = v[j] * inv;
   }
 }
@@ -142,9 +167,10 @@ extern "C" int zf_short_conv(const void* src, int dtype, long long src_stride, c
       (size_t)unit_heads * hd > (size_t)C || scaled_heads > unit_heads || n_seqs < 1 ||
       (single_tokens && T != n_seqs) || hd > DL_CONV_THREADS * DL_CONV_PER_THREAD)
     return -2;
-  // whole heads a block where a head fits a workgroup, else one head a block
-  const int hpb = hd <= DL_CONV_THREADS ? DL_CONV_THREADS / hd : 0;
-  const int head_blocks = unit_heads == 0 ? 0 : (hpb > 0 ? (unit_heads + hpb - 1) / hpb : unit_heads);
+  // a head takes whole waves (one, two or four): as many heads a block as fit
+  const int hw = hd > 128 ? 4 : (hd > 64 ? 2 : 1);
+  const int hpb = DL_CONV_THREADS / (hw * ZF_WAVE);
+  const int head_blocks = (unit_heads + hpb - 1) / hpb;
   const int plain = C - unit_heads * hd;
   const dim3 grid(T, head_blocks + (plain + DL_CONV_THREADS - 1) / DL_CONV_THREADS);
   const dim3 sgrid(n_seqs, (C + DL_CONV_THREADS - 1) / DL_CONV_THREADS);
@@ -166,21 +192,6 @@ extern "C" int zf_short_conv(const void* src, int dtype, long long src_stride, c
 #define DL_MAX_LANES 16        // lanes that share a column's key channels
 #define DL_PF 4                // 16-byte pieces of q and of k, and values of v, a thread fetches ahead
 
-// The sum over the CG lanes (a power of two up to 16, aligned in a row of 16 lanes) that share a
-// column, in every one of them, through the data-parallel lane moves: neighbours, pairs, then the
-// mirrored half row and row (a lane and its mirror hold sums over different halves).
-template <int CTRL>
-__device__ __forceinline__ float dl_move(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float dl_lanes_sum(float v, int CG) {
-  if (CG >= 2) v += dl_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
-  if (CG >= 4) v += dl_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
-  if (CG >= 8) v += dl_move<0x141>(v);     // row_half_mirror
-  if (CG >= 16) v += dl_move<0x140>(v);    // row_mirror
-  return v;
-}
-
 // A thread holds R key channels of one value column of S; CG lanes side by side hold the
 // column's P = CG * R channels (zeros beyond d).  A request's matrices lie [head][column][P] in
 // its state, so a thread's channels are consecutive.  Grid (column tiles, heads, sequences).
@@ -189,14 +200,15 @@ __device__ __forceinline__ float dl_lanes_sum(float v, int CG) {
 // Sixteen tokens at a time lie in LDS; the next sixteen are asked for before these are walked
 // (16-byte pieces, where the rows' offsets allow: VEC), and a token's operands are read from LDS
 // while the token before it is computed.
-template <int R, bool VEC>
+template <int R, int CG, bool VEC>
 __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ qkv, int C, int q_off, int k_off, int v_off,
     const float* __restrict__ ab, const float* __restrict__ a_log,
     const float* __restrict__ dt_bias, float* __restrict__ state, long long state_stride,
     const int* __restrict__ state_slots, const int* __restrict__ q_start, float* __restrict__ out,
-    int H, int KH, int d, int dv, int CG, int cols) {
-#pragma clang fp contract(off)
+    int H, int KH, int d, int dv, int cols) {
+  // (fused multiply-adds as the compiler forms them: this one kernel walks every portion, whole
+  // prompt or single token, so every cut of a sequence gets the same instructions)
   extern __shared__ float lds[];
   const int P = CG * R;
   float* qs = lds;                          // [DL_STAGE][P]
@@ -223,7 +235,6 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   }
   const float decay_rate = expf(a_log[h]);
   const float dtb = dt_bias[h];
-  const int wave = tid / ZF_WAVE, lane = tid % ZF_WAVE, nwaves = (nthreads + ZF_WAVE - 1) / ZF_WAVE;
   const int P4 = P / 4;
   // what a thread fetches ahead: pieces tid, tid + nthreads, ... of the stage's q and k rows,
   // one value of its v columns, and (the first threads) a token's two numbers
@@ -303,15 +314,17 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     stage(t0, n);
     __syncthreads();
     if (t0 + DL_STAGE < len) fetch(t0 + DL_STAGE, min(DL_STAGE, len - t0 - DL_STAGE));
-    for (int tok = wave; tok < n; tok += nwaves) {
+    // q . k of every staged token: sixteen lanes a token
+    for (int tok = tid / 16; tok < n; tok += nthreads / 16) {
       float dot = 0.f;
-      for (int c = lane; c < P; c += ZF_WAVE) dot += qs[tok * P + c] * ks[tok * P + c];
-      dot = wave_sum(dot);
-      if (lane == 0) ds[tok] = dot;
+      for (int c = tid % 16; c < P; c += 16) dot += qs[tok * P + c] * ks[tok * P + c];
+      dot = dl_lanes_sum<16>(dot);
+      if (tid % 16 == 0) ds[tok] = dot;
     }
     __syncthreads();
     // a token's operands are read a token ahead
     float kk[R], qq[R], g, b, v, qk;
+    float* o_at = out + (size_t)(first + t0) * H * dv + (size_t)h * dv + (live ? col : 0);
     auto read = [&](int tok) {
       const float* qrow = qs + tok * P + cg * R;
       const float* krow = ks + tok * P + cg * R;
@@ -336,12 +349,12 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
       }
       const float gc = g, bc = b, vc = v, qkc = qk;
       if (tok + 1 < n) read(tok + 1);
-      const float rs = dl_lanes_sum(r0 + r1, CG), ps = dl_lanes_sum(p0 + p1, CG);
+      const float rs = dl_lanes_sum<CG>(r0 + r1), ps = dl_lanes_sum<CG>(p0 + p1);
       const float w = bc * (vc - gc * rs);
 #pragma unroll
       for (int r = 0; r < R; ++r) S[r] = gc * S[r] + kc[r] * w;
-      if (live && cg == 0)
-        out[(size_t)(first + t0 + tok) * H * dv + (size_t)h * dv + col] = gc * ps + qkc * w;
+      if (live && cg == 0) *o_at = gc * ps + qkc * w;
+      o_at += (size_t)H * dv;
     }
   }
   if (live) {
@@ -371,20 +384,23 @@ extern "C" int zf_delta_recurrence(const float* qkv, int C, int q_off, int k_off
                    ((uintptr_t)qkv % 16) == 0 &&
                    DL_STAGE * (R * CG / 4) <= DL_PF * threads && DL_STAGE * cols <= DL_PF * threads &&
                    DL_STAGE <= threads;
-#define DL_REC_LAUNCH(RR)                                                                        \
-  if (vec)                                                                                       \
-    hipLaunchKernelGGL((delta_recurrence_kernel<RR, true>), grid, block, smem, stream, qkv, C,   \
-                       q_off, k_off, v_off, ab, a_log, dt_bias, state, state_stride,             \
-                       state_slots, q_start, out, H, KH, d, dv, CG, cols);                       \
-  else                                                                                           \
-    hipLaunchKernelGGL((delta_recurrence_kernel<RR, false>), grid, block, smem, stream, qkv, C,  \
-                       q_off, k_off, v_off, ab, a_log, dt_bias, state, state_stride,             \
-                       state_slots, q_start, out, H, KH, d, dv, CG, cols)
-  switch (R) {
-    case 8: DL_REC_LAUNCH(8); break;
-    case 12: DL_REC_LAUNCH(12); break;
-    case 16: DL_REC_LAUNCH(16); break;
-    default: return -2;
+#define DL_REC_LAUNCH(RR, GG)                                                                    \
+  if (R == RR && CG == GG) {                                                                     \
+    if (vec)                                                                                     \
+      hipLaunchKernelGGL((delta_recurrence_kernel<RR, GG, true>), grid, block, smem, stream,     \
+                         qkv, C, q_off, k_off, v_off, ab, a_log, dt_bias, state, state_stride,   \
+                         state_slots, q_start, out, H, KH, d, dv, cols);                         \
+    else                                                                                         \
+      hipLaunchKernelGGL((delta_recurrence_kernel<RR, GG, false>), grid, block, smem, stream,    \
+                         qkv, C, q_off, k_off, v_off, ab, a_log, dt_bias, state, state_stride,   \
+                         state_slots, q_start, out, H, KH, d, dv, cols);                         \
+    launched = true;                                                                             \
   }
+  bool launched = false;
+  // (the padded key sizes 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+  DL_REC_LAUNCH(8, 1) DL_REC_LAUNCH(12, 1) DL_REC_LAUNCH(8, 2) DL_REC_LAUNCH(12, 2)
+  DL_REC_LAUNCH(8, 4) DL_REC_LAUNCH(12, 4) DL_REC_LAUNCH(8, 8) DL_REC_LAUNCH(12, 8)
+  DL_REC_LAUNCH(8, 16) DL_REC_LAUNCH(12, 16) DL_REC_LAUNCH(16, 16)
+  if (!launched) return -2;
   ZF_CHECK_LAUNCH();
 }
