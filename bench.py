@@ -1296,15 +1296,15 @@ def main_nupovik(args) -> int:
 # design with a recurrence (its gated linear attention at the same heads).
 def _kg_moe(experts, identity, top, ff, groups, shared):
     return {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": shared},
-            "router": {"experts": experts, "identity": identity, "top": top, "scale": 2.0,
+            "router": {"experts": experts, "identity": identity, "top": top, "scale": 2.5,
                        "groups": {"count": groups[0], "keep": groups[1]}}}
 
 
 def _kg_mixer(heads, kv, r_heads, r_kv):
     return {"left": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128,
-                     "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 500000.0}},
+                     "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 1000000.0}},
             "right": {"heads": r_heads, "kv_heads": r_kv, "dim": 128, "vdim": 128, "conv": 4},
-            "left_scale": 0.8, "right_scale": 0.9}
+            "left_scale": 0.75, "right_scale": 1.25}
 
 
 KUGISUN_SHAPES = {
@@ -1408,7 +1408,7 @@ def kugisun_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float
     qkv = rnd(rows, (nH + 2 * nKV) * hd)
     bias = rnd32((nH + 2 * nKV) * hd)
     gq, gk = torch.ones(hd, device=dev), torch.ones(hd, device=dev)
-    freq = torch.tensor([500000.0 ** (-2.0 * i / 64) for i in range(32)], device=dev)
+    freq = torch.tensor([1000000.0 ** (-2.0 * i / 64) for i in range(32)], device=dev)
     qw, kw = nH * hd, nKV * hd
     segs = [ops.RowSegment(0, qw, o, gain=gq, eps=1e-6, hd=hd, bias=bias[:qw].contiguous(),
                            per_head=True, rot_dims=64, freq=freq, interleaved=True),
@@ -1488,7 +1488,7 @@ def kugisun_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float
     bco, aco = torch.ones(S, device=dev), torch.ones(S, device=dev) / S
     gw = torch.ones(W, device=dev)
     hout = torch.empty((rows, W), dtype=bf, device=dev)
-    t_new = _timed_graph(lambda: ops.streams_step(x, [(y0, 0.8), (y1, 1.0)], M, bco, read=True,
+    t_new = _timed_graph(lambda: ops.streams_step(x, [(y0, 0.75), (y1, 1.0)], M, bco, read=True,
                                                   in_coef=aco, gain=gw, eps=1e-6, out=hout))
     x1 = torch.randn((rows, W), generator=g, device=dev)
     t_old = _timed_graph(lambda: ops.rmsnorm(x1, gw, 1e-6, hout))
@@ -1525,7 +1525,7 @@ def kugisun_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float
 
     def mixture():
         ops.moe_route(h, router, None, ids, share, scoring="softmax_all", correction=correction,
-                      groups=groups, group_mark=1, normalize=False, weight_scale=2.0, extra=sgate)
+                      groups=groups, group_mark=1, normalize=False, weight_scale=2.5, extra=sgate)
         ops.moe_experts(h, gu, down, ids, share, y, branch, 0.0, 1.0, 0.0, add=False, n_identity=I)
         ops.gemm(h, wsgu, sgu, w_tiled=True)
         ops.gated_act(sgu, sy, 0.0, 1.0, 0.0, row_factor=sgate[:, 0])
