@@ -85,8 +85,8 @@ KG_C = {"architecture": "Kugisun", "vocab": 97, "width": 50, "max_positions": 25
 
 # widths the bfloat16 matrix kernels take, heads the MFMA attention kernels take; key sizes of 64
 # and 128 for the delta rule; four copies; two outputs that hand their input on
-_D1 = _layer(_left(4, 2, 64, 64, 0.12, (32, 250000.0)), _right(4, 2, 64, 64, 4), 0.75, 1.25,
-             _moe(10, 3, 64, identity=2, groups=(4, 2), scale=1.5, shared=192))
+_D1 = _layer(_left(4, 2, 64, 64, 0.12, (32, 250000.0)), _right(4, 2, 64, 64, 4), 1.1, 0.7,
+             _moe(6, 3, 64, identity=2, groups=(4, 2), scale=1.5, shared=192))
 KG_D = {"architecture": "Kugisun", "vocab": 512, "width": 128, "max_positions": 1024, "streams": 4,
         "norm": {"eps": 1e-6},
         "layers": [_layer(_left(2, 2, 128, 128, 0.09, (128, 10000.0)), _right(2, 1, 128, 32, 4),
