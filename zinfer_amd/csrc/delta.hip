@@ -23,7 +23,7 @@ __device__ __forceinline__ float dl_softplus(float z) {
   return z > 20.f ? z : log1pf(expf(z));
 }
 
-// The sum over the CG lanes (a power of two up to 16, aligned in a row of 16 lanes) that share a
+// The sum over the CG lanes (a power of two up to 64, aligned) that share a
 // column, in every one of them, through the data-parallel lane moves: neighbours, pairs, then the
 // mirrored half row and row (a lane and its mirror hold sums over different halves).
 template <int CTRL>
@@ -38,6 +38,17 @@ __device__ __forceinline__ float dl_lanes_sum(float v) {
   if constexpr (CG >= 4) v += dl_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
   if constexpr (CG >= 8) v += dl_move<0x141>(v);     // row_half_mirror
   if constexpr (CG >= 16) v += dl_move<0x140>(v);    // row_mirror
+  if constexpr (CG >= 32) {
+    // rows of 16 lanes in pairs: one copy takes its odd rows from the other's even rows and
+    // gives its own odd rows for them, so the two copies hold a pair's two rows lane by lane
+    typedef unsigned int dl_u2 __attribute__((ext_vector_type(2)));
+    const dl_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r.x) + __uint_as_float(r.y);
+    if constexpr (CG >= 64) {
+      const dl_u2 q = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+      v = __uint_as_float(q.x) + __uint_as_float(q.y);      // the wave's two halves
+    }
+  }
   return v;
 }
 
@@ -189,7 +200,7 @@ extern "C" int zf_short_conv(const void* src, int dtype, long long src_stride, c
 
 // ------------------------------------------------------------------ the recurrence
 #define DL_STAGE 16            // tokens staged in LDS at a time
-#define DL_MAX_LANES 16        // lanes that share a column's key channels
+#define DL_MAX_LANES 64        // lanes that share a column's key channels
 #define DL_PF 4                // 16-byte pieces of q and of k, and values of v, a thread fetches ahead
 
 // A thread holds R key channels of one value column of S; CG lanes side by side hold the
@@ -217,6 +228,7 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   float* gs = vs + DL_STAGE * cols;         // [DL_STAGE] decay
   float* bs = gs + DL_STAGE;                // [DL_STAGE] step size
   float* ds = bs + DL_STAGE;                // [DL_STAGE] q . k
+  float* os = ds + DL_STAGE;                // [DL_STAGE][cols] the stage's outputs
   const int h = blockIdx.y, seq = blockIdx.z;
   const int kh = h / (H / KH);
   const int first = q_start[seq], len = q_start[seq + 1] - first;
@@ -228,10 +240,18 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   float* S_mem = state + (size_t)state_slots[seq] * state_stride
                  + ((size_t)h * dv + (live ? col : 0)) * P + cg * R;
   float S[R];
+  if constexpr (R % 4 == 0) {
 #pragma unroll
-  for (int r = 0; r < R; r += 4) {
-    const float4 v = live ? *(const float4*)(S_mem + r) : make_float4(0.f, 0.f, 0.f, 0.f);
-    S[r] = v.x; S[r + 1] = v.y; S[r + 2] = v.z; S[r + 3] = v.w;
+    for (int r = 0; r < R; r += 4) {
+      const float4 v = live ? *(const float4*)(S_mem + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+      S[r] = v.x; S[r + 1] = v.y; S[r + 2] = v.z; S[r + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; r += 2) {
+      const float2 v = live ? *(const float2*)(S_mem + r) : make_float2(0.f, 0.f);
+      S[r] = v.x; S[r + 1] = v.y;
+    }
   }
   const float decay_rate = expf(a_log[h]);
   const float dtb = dt_bias[h];
@@ -324,16 +344,26 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     __syncthreads();
     // a token's operands are read a token ahead
     float kk[R], qq[R], g, b, v, qk;
-    float* o_at = out + (size_t)(first + t0) * H * dv + (size_t)h * dv + (live ? col : 0);
+
     auto read = [&](int tok) {
       const float* qrow = qs + tok * P + cg * R;
       const float* krow = ks + tok * P + cg * R;
+      if constexpr (R % 4 == 0) {
 #pragma unroll
-      for (int r = 0; r < R; r += 4) {
-        const float4 kv = *(const float4*)(krow + r);
-        const float4 qv = *(const float4*)(qrow + r);
-        kk[r] = kv.x; kk[r + 1] = kv.y; kk[r + 2] = kv.z; kk[r + 3] = kv.w;
-        qq[r] = qv.x; qq[r + 1] = qv.y; qq[r + 2] = qv.z; qq[r + 3] = qv.w;
+        for (int r = 0; r < R; r += 4) {
+          const float4 kv = *(const float4*)(krow + r);
+          const float4 qv = *(const float4*)(qrow + r);
+          kk[r] = kv.x; kk[r + 1] = kv.y; kk[r + 2] = kv.z; kk[r + 3] = kv.w;
+          qq[r] = qv.x; qq[r + 1] = qv.y; qq[r + 2] = qv.z; qq[r + 3] = qv.w;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; r += 2) {
+          const float2 kv = *(const float2*)(krow + r);
+          const float2 qv = *(const float2*)(qrow + r);
+          kk[r] = kv.x; kk[r + 1] = kv.y;
+          qq[r] = qv.x; qq[r + 1] = qv.y;
+        }
       }
       g = gs[tok]; b = bs[tok]; v = vs[tok * cols + col_l]; qk = ds[tok];
     };
@@ -353,14 +383,25 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
       const float w = bc * (vc - gc * rs);
 #pragma unroll
       for (int r = 0; r < R; ++r) S[r] = gc * S[r] + kc[r] * w;
-      if (live && cg == 0) *o_at = gc * ps + qkc * w;
-      o_at += (size_t)H * dv;
+      if (cg == 0) os[tok * cols + col_l] = gc * ps + qkc * w;
+    }
+    // the stage's outputs leave side by side (the next stage's barrier stands between these
+    // reads and the next writes)
+    __syncthreads();
+    for (int i = tid; i < n * cols; i += nthreads) {
+      const int tok = i / cols, c = blockIdx.x * cols + i % cols;
+      if (c < dv) out[(size_t)(first + t0 + tok) * H * dv + (size_t)h * dv + c] = os[i];
     }
   }
   if (live) {
+    if constexpr (R % 4 == 0) {
 #pragma unroll
-    for (int r = 0; r < R; r += 4)
-      *(float4*)(S_mem + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+      for (int r = 0; r < R; r += 4)
+        *(float4*)(S_mem + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; r += 2) *(float2*)(S_mem + r) = make_float2(S[r], S[r + 1]);
+    }
   }
 }
 
@@ -378,7 +419,7 @@ extern "C" int zf_delta_recurrence(const float* qkv, int C, int q_off, int k_off
       ZF_WAVE % CG != 0)
     return -2;
   const dim3 grid((dv + cols - 1) / cols, H, n_seqs), block(threads);
-  const size_t smem = (size_t)(DL_STAGE * (2 * R * CG + cols) + 3 * DL_STAGE) * sizeof(float);
+  const size_t smem = (size_t)(DL_STAGE * (2 * R * CG + 2 * cols) + 3 * DL_STAGE) * sizeof(float);
   // 16-byte pieces: every row offset a multiple of four floats, and few enough pieces a thread
   const bool vec = C % 4 == 0 && q_off % 4 == 0 && k_off % 4 == 0 && d % 4 == 0 &&
                    ((uintptr_t)qkv % 16) == 0 &&
